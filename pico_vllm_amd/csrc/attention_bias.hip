@@ -91,7 +91,7 @@ extern "C" int pico_kv_mix_store(const void* qkv, int dtype, int ld, int k_col, 
 // The plain kernel.  Keys are visited in blocks of 64 aligned to absolute positions, so the result at a position does
 // not depend on how the sequence was cut into steps.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int NV>
 __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ positions,
@@ -111,7 +111,9 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) acc[i] = 0.f;
   // blocks of 64 keys aligned to absolute positions: first those that hold kept first positions in front of the
   // window, then the window's; a block that holds both is visited once
   const int keep = bp.window > 0 ? min(bp.keep_first, lo) : 0;      // keys below `keep` are seen although the window has passed them
@@ -138,7 +140,9 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     __syncthreads();
     ps[lane] = p;
     __syncthreads();
-    float blk[4] = {0.f, 0.f, 0.f, 0.f};
+    float blk[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) blk[i] = 0.f;
     const int kend = min(64, pos - c0 + 1);
     for (int kk = 0; kk < kend; kk++) {
       const int kpos = c0 + kk;
@@ -148,18 +152,18 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
       const T* vp = v_cache + ((size_t)page * nkv + g) * dv * P + kpos % P;
       const float pk = ps[kk];
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
+      for (int i = 0; i < NV; i++) {
         const int dim = lane + 64 * i;
         if (dim < dv) blk[i] = fmaf(pk, load_f32(vp + (size_t)dim * P), blk[i]);
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[i] = fmaf(acc[i], alpha, blk[i]);
+    for (int i = 0; i < NV; i++) acc[i] = fmaf(acc[i], alpha, blk[i]);
     m = m_new;
   }
   T* o = out + ((size_t)t * nq + h) * dv;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < NV; i++) {
     const int dim = lane + 64 * i;
     if (dim >= dv) continue;
     float v = acc[i] / l;
@@ -177,7 +181,7 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
   PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && dk > 0 && dv > 0 && P > 0 && max_pages > 0 && num_pages > 0,
                "pico_attn_bias_plain: bad sizes");
   PICO_REQUIRE(nq % nkv == 0, "pico_attn_bias_plain: %d query heads are not a multiple of %d kv heads", nq, nkv);
-  PICO_REQUIRE(dk <= 1024 && dv <= 256, "pico_attn_bias_plain: key size %d (at most 1024) or value size %d (at most 256) too large", dk, dv);
+  PICO_REQUIRE(dk <= 1024 && dv <= 512, "pico_attn_bias_plain: key size %d (at most 1024) or value size %d (at most 512) too large", dk, dv);
   PICO_REQUIRE(nq <= 65535, "pico_attn_bias_plain: too many heads");
   PICO_REQUIRE(q_stride >= nq * dk, "pico_attn_bias_plain: query row stride too small");
   PICO_REQUIRE(window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attn_bias_plain: window, interval and span must not be negative");
@@ -187,14 +191,26 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
   const BiasParams bp{scale, temp_coef, slope_span, temp_every, window, softcap, keep_first};
   dim3 grid(T, nq);
   const size_t lds = (size_t)(dk + 64) * sizeof(float);
-  if (dtype == PICO_DTYPE_F32)
-    attn_bias_plain_kernel<float><<<grid, 64, lds, stream>>>(
-        (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
-        token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
-  else if (dtype == PICO_DTYPE_BF16)
-    attn_bias_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>(
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
-        token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
+  if (dtype == PICO_DTYPE_F32) {
+    if (dv <= 256)
+      attn_bias_plain_kernel<float, 4><<<grid, 64, lds, stream>>>(
+          (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
+          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
+    else
+      attn_bias_plain_kernel<float, 8><<<grid, 64, lds, stream>>>(
+          (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
+          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
+  }
+  else if (dtype == PICO_DTYPE_BF16) {
+    if (dv <= 256)
+      attn_bias_plain_kernel<bf16_t, 4><<<grid, 64, lds, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
+          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
+    else
+      attn_bias_plain_kernel<bf16_t, 8><<<grid, 64, lds, stream>>>(
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
+          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
+  }
   else
     PICO_REQUIRE(false, "pico_attn_bias_plain: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

@@ -78,8 +78,12 @@ __global__ __launch_bounds__(TB == 16 ? 256 : 512) void gla_scan_kernel(const T*
                                                        float* __restrict__ out, int H, int dk, int dv, float qscale,
                                                        int num_slots, int chunk, int max_chunks, float* __restrict__ ws,
                                                        float* __restrict__ ws_decay, const T* __restrict__ a2,
-                                                       const float* __restrict__ a2_bias, int a_col, int R, float inv_tau) {
+                                                       const float* __restrict__ a2_bias, int a_col, int R, float inv_tau,
+                                                       const float* __restrict__ head_decay) {
   extern __shared__ float lds[];
+  // head_decay given: every key channel of head h decays by the constant head_decay[h] at every token (log_decay, a2
+  // are not read); the decay is multiplied in as it is, no logarithm and exponential between
+  const float fixed = head_decay ? head_decay[blockIdx.y] : 0.f;
   const int nw = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int CP = nw * GLA_CPT;                          // key channels with padding
   float* qs = lds;                                      // [TB][CP]
@@ -125,7 +129,9 @@ __global__ __launch_bounds__(TB == 16 ? 256 : 512) void gla_scan_kernel(const T*
     // the chunk's decays multiplied up, as the sum of their logarithms, for the walk over the chunks
     for (int c = threadIdx.x; c < dk; c += blockDim.x) {
       float sum = 0.f;
-      for (int t = t_begin; t < t_end; t++) sum += log_decay[(size_t)t * H * dk + (size_t)h * dk + c];
+      if (head_decay) sum = (float)(t_end - t_begin) * logf(fixed);
+      else
+        for (int t = t_begin; t < t_end; t++) sum += log_decay[(size_t)t * H * dk + (size_t)h * dk + c];
       ws_decay[((size_t)blockIdx.x * H + h) * dk + c] = sum;
     }
   }
@@ -144,7 +150,9 @@ __global__ __launch_bounds__(TB == 16 ? 256 : 512) void gla_scan_kernel(const T*
       const T* row = x + (size_t)(t0 + tt) * ldx + (size_t)h * dk + c_in;
       rq[j] = MODE != GLA_LOCAL ? row[q_col] : row[k_col];
       rk[j] = row[k_col];
-      if (!FUSED) {
+      if (head_decay) {
+        ra[j] = 0.f;
+      } else if (!FUSED) {
         ra[j] = log_decay[(size_t)(t0 + tt) * H * dk + (size_t)h * dk + c_in];
       } else if (tt0 + 2 * j >= nb) {
         ra[j] = 0.f;                                    // no such token in this block: nothing to work out
@@ -173,7 +181,7 @@ __global__ __launch_bounds__(TB == 16 ? 256 : 512) void gla_scan_kernel(const T*
       const bool in = tt < nb && c < dk;
       qs[i] = (in && MODE != GLA_LOCAL) ? load_f32(&rq[j]) * qscale : 0.f;
       ks[i] = in ? load_f32(&rk[j]) : 0.f;
-      as[i] = in ? expf(ra[j]) : 1.f;
+      as[i] = in ? (head_decay ? fixed : expf(ra[j])) : 1.f;
     }
     float vv[VPL][TB];
 #pragma unroll
@@ -269,8 +277,8 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
                              const int* cu_seqlens, const int* state_slots, float* state, float* out, int num_seqs,
                              int T, int H, int dk, int dv, float qscale, int num_slots, int chunk, int max_chunks,
                              float* ws, float* ws_decay, const void* a2, const float* a2_bias, int a_col, int R, float tau,
-                             hipStream_t stream) {
-  PICO_REQUIRE(log_decay != nullptr || (chunk == 0 && a2 != nullptr && R > 0 && a_col >= 0 && ldx >= a_col + R && tau > 0.f),
+                             const float* head_decay, hipStream_t stream) {
+  PICO_REQUIRE(head_decay != nullptr || log_decay != nullptr || (chunk == 0 && a2 != nullptr && R > 0 && a_col >= 0 && ldx >= a_col + R && tau > 0.f),
                "pico_gla_scan: without the decays' logarithms the walk needs what makes them, and runs whole");
   PICO_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && dk > 0 && dv > 0 && num_slots > 0, "pico_gla_scan: bad sizes");
   PICO_REQUIRE(dk <= 8 * GLA_CPT, "pico_gla_scan: at most %d key channels a head, got %d", 8 * GLA_CPT, dk);
@@ -293,11 +301,11 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
   const int vb = (dv + 64 * vpl - 1) / (64 * vpl);
 #define GLA_ARGS(TT)                                                                                                       \
   (const TT*)x, ldx, q_col, k_col, v_col, log_decay, cu_seqlens, state_slots, state, out, H, dk, dv, qscale, num_slots,   \
-      chunk, max_chunks, ws, ws_decay, (const TT*)a2, a2_bias, a_col, R, 1.0f / (tau > 0.f ? tau : 1.f)
+      chunk, max_chunks, ws, ws_decay, (const TT*)a2, a2_bias, a_col, R, 1.0f / (tau > 0.f ? tau : 1.f), head_decay
 #define GLA_LAUNCH(TT, MODE, GX)                                                                                           \
   do {                                                                                                                     \
     constexpr bool fused = MODE == GLA_WHOLE;     /* with FUSED the launch below is taken only when log_decay is null */ \
-    if (log_decay == nullptr && fused) {                                                                                   \
+    if (log_decay == nullptr && head_decay == nullptr && fused) {                                                                                   \
       if (tb == 16)                                                                                                        \
         gla_scan_kernel<TT, MODE, 16, 1, fused><<<dim3(GX, H, vb), 64 * nw, lds, stream>>>(GLA_ARGS(TT));                  \
       else                                                                                                                 \

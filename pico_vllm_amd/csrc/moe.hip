@@ -351,3 +351,62 @@ extern "C" int pico_moe_experts_plain(const void* h, int ldh, int dtype, const v
   PICO_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// A third way of choosing: logits z = x Wr^T + bias; the `top` largest logits are chosen (the lowest index among equal
+// ones) and the weights are the softmax over the chosen logits only.  Wr may hold `extra` rows behind the E experts'
+// whose logits are made in the same launch and take no part in the choice (a gate of the layer, say): z is
+// [T, E + extra], and what the choice reads of it has the bias added.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void moe_route_top_softmax_kernel(float* __restrict__ z, const float* __restrict__ bias,
+                                                                   int T, int E, int ldz, int top,
+                                                                   int* __restrict__ experts, float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  float* row = z + (size_t)t * ldz;
+  if (bias)
+    for (int e = 0; e < E; e++) row[e] += bias[e];
+  int chosen[MOE_MAX_TOP];
+  float val[MOE_MAX_TOP];
+  for (int k = 0; k < top; k++) {
+    int best = -1;
+    float bz = 0.f;
+    for (int e = 0; e < E; e++) {
+      bool taken = false;
+      for (int j = 0; j < k; j++) taken |= chosen[j] == e;
+      if (taken) continue;
+      const float v = row[e];
+      if (best < 0 || v > bz) { best = e; bz = v; }
+    }
+    chosen[k] = best;
+    val[k] = bz;
+  }
+  const float largest = val[0];
+  float sum = 0.f;
+  for (int k = 0; k < top; k++) { val[k] = expf(val[k] - largest); sum += val[k]; }
+  for (int k = 0; k < top; k++) {
+    experts[(size_t)t * top + k] = chosen[k];
+    weights[(size_t)t * top + k] = val[k] / sum;
+  }
+}
+
+extern "C" int pico_moe_router_top_softmax(const void* x, int ldx, int dtype, const float* Wr, const float* bias, int T,
+                                           int E, int extra, int D, int top, float* z, int* experts, float* weights,
+                                           hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && E > 0 && extra >= 0 && D > 0 && ldx >= D && top > 0 && top <= E && top <= MOE_MAX_TOP,
+               "pico_moe_router_top_softmax: %d of %d experts per token is outside what the kernel takes (at most %d)", top, E, MOE_MAX_TOP);
+  PICO_REQUIRE(dtype == PICO_DTYPE_F32 || dtype == PICO_DTYPE_BF16, "pico_moe_router_top_softmax: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  const int rows = E + extra;
+  const dim3 grid((T + ROUTER_TOKENS - 1) / ROUTER_TOKENS, (rows + 3) / 4);
+  PICO_REQUIRE(grid.y <= 65535, "pico_moe_router_top_softmax: too many experts");
+  const size_t esz = dtype == PICO_DTYPE_F32 ? 4 : 2;
+  const bool vec = D % 4 == 0 && ldx % 4 == 0 && (uintptr_t)x % (4 * esz) == 0 && (uintptr_t)Wr % 16 == 0;
+#define LAUNCH(TT, V) moe_logits_kernel<TT, V><<<grid, 256, 0, stream>>>((const TT*)x, ldx, Wr, T, rows, D, z)
+  if (dtype == PICO_DTYPE_F32) { if (vec) LAUNCH(float, true); else LAUNCH(float, false); }
+  else { if (vec) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
+#undef LAUNCH
+  moe_route_top_softmax_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, bias, T, E, rows, top, experts, weights);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

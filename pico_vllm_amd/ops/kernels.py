@@ -715,7 +715,8 @@ GLA_MAX_KEY_DIM = 256
 
 def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: Optional[torch.Tensor], cu_seqlens: torch.Tensor,
              state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, dk: int, dv: int,
-             qscale: float, chunk: int = 0, decay_from: Optional[tuple] = None) -> torch.Tensor:
+             qscale: float, chunk: int = 0, decay_from: Optional[tuple] = None,
+             head_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The recurrence S <- diag(exp(log_decay_t)) S + k_t v_t^T, o_t = S^T q_t qscale, for every sequence of the step from
     its state slot (``state`` float32 [slots, heads, dk, dv], updated in place).  Returns o float32 [T, heads * dv].
     ``chunk`` > 0: sequences are cut into chunks of that many tokens that run side by side (every chunk from zero, a walk
@@ -727,7 +728,12 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: Opt
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < max(q_col + heads * dk, k_col + heads * dk, v_col + heads * dv):
         raise KernelError("gla_scan: x must be [T, columns] with unit stride along the row and hold q, k and v")
     a_col, a2, a2_bias, tau, R = 0, None, None, 0.0, 0
-    if log_decay is None:
+    if head_decay is not None:
+        # one constant decay a head (float32 [heads], the decays themselves): no logarithms are read or made
+        _gpu(head_decay)
+        if log_decay is not None or head_decay.dtype != torch.float32 or tuple(head_decay.shape) != (heads,) or not head_decay.is_contiguous():
+            raise KernelError(f"gla_scan: a fixed decay is contiguous float32 [{heads}] and comes without logarithms")
+    elif log_decay is None:
         if chunk or decay_from is None:
             raise KernelError("gla_scan: without the decays' logarithms the walk runs whole and needs what makes them")
         a_col, a2, a2_bias, tau = decay_from
@@ -756,7 +762,7 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: Opt
     _check(lib, lib.pico_gla_scan(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), q_col, k_col, v_col, _ptr(log_decay),
                                   _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out), num_seqs, T, heads, dk, dv,
                                   c_float(qscale), state.shape[0], chunk, max_chunks, _ptr(ws), _ptr(ws_decay), _ptr(a2),
-                                  _ptr(a2_bias), a_col, R, c_float(tau), _stream()))
+                                  _ptr(a2_bias), a_col, R, c_float(tau), _ptr(head_decay), _stream()))
     return out
 
 
@@ -944,3 +950,233 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, expe
                                              _ptr(sorted_rows), _ptr(tile_expert), tiles, _ptr(y), _ptr(out), T, top, E, F,
                                              D, c_float(limit), c_float(alpha), mode, _stream()))
     return out[0] if top == 1 else out
+
+
+# ---- layer norm, scaled sums, the embedding of token pairs ---------------------------------------------------------
+LN_MAX_SLABS = 16
+
+
+def _delta_args(resid, delta, who):
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    slabs = 1
+    if delta is not None:
+        if delta.dim() == 3:
+            slabs = delta.shape[0]
+            if delta.dtype != torch.float32:
+                raise KernelError("a stack of partial sums must be float32")
+        if tuple(delta.shape[-2:]) != (T, H) or not delta.is_contiguous():
+            raise KernelError(f"{who}: delta must be contiguous and shaped like the residual stream")
+    return T, H, slabs
+
+
+def _vec(t, H, name):
+    if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != (H,) or not t.is_contiguous()):
+        raise KernelError(f"{name} must be contiguous float32 [{H}]")
+
+
+def add_layernorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor, eps: float,
+                  out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                  delta_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Layer norm (weight and bias, the variance from the deviations) of resid + delta_scale * delta.
+    rows is None: resid is updated in place and every row normed; rows given: only those rows, resid left alone.
+    delta: [T, H], or a float32 stack [S, T, H] whose slabs are added up first; delta_scale: float32 [H] or None (ones)."""
+    _gpu(resid, delta, weight, bias, rows, delta_scale)
+    T, H, slabs = _delta_args(resid, delta, "add_layernorm")
+    _vec(weight, H, "norm weight"); _vec(bias, H, "norm bias"); _vec(delta_scale, H, "delta scale")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    out = torch.empty(n, H, dtype=out_dtype, device=resid.device)
+    lib = library.core()
+    _check(lib, lib.pico_add_layernorm(_ptr(resid), _ptr(delta), _dt(delta) if delta is not None else F32, slabs, c_ll(T * H),
+                                       _ptr(delta_scale), _ptr(weight), _ptr(bias), _ptr(out), _DT[out_dtype], _ptr(rows), n, H,
+                                       c_float(eps), _stream()))
+    return out
+
+
+def scaled_add(resid: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.Tensor] = None,
+               gate: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """resid (float32 [T, H], in place) += scale * (a + sigmoid(gate) * b).  a: [T, H] or a float32 stack [S, T, H];
+    b: [T, H]; gate: float32 logits, one a row (a column of a wider float32 matrix will do); scale float32 [H] or None."""
+    _gpu(resid, a, b, gate, scale)
+    T, H, slabs = _delta_args(resid, a, "scaled_add")
+    _vec(scale, H, "scale")
+    if b is not None and (tuple(b.shape) != (T, H) or not b.is_contiguous()):
+        raise KernelError("scaled_add: b must be contiguous and shaped like the residual stream")
+    gs = 0
+    if gate is not None:
+        if b is None or gate.dtype != torch.float32 or gate.shape[0] != T or gate.dim() > 2 or (gate.dim() == 2 and gate.shape[1] != 1):
+            raise KernelError("scaled_add: the gate is float32 [T] or [T, 1] and goes with b")
+        gs = gate.stride(0) if T > 1 else 1
+    lib = library.core()
+    _check(lib, lib.pico_scaled_add(_ptr(resid), _ptr(a), _dt(a) if a is not None else F32, slabs, c_ll(T * H), _ptr(b),
+                                    _dt(b) if b is not None else F32, _ptr(gate), gs, _ptr(scale), T, H, _stream()))
+    return resid
+
+
+def pair_embed(resid: torch.Tensor, table: torch.Tensor, ctx, last: torch.Tensor, mul_prev: int, mul_cur: int, buckets: int) -> torch.Tensor:
+    """resid[t] += table[(previous token * mul_prev + token * mul_cur) mod buckets], at position 0 table[buckets].
+    ``last`` int32 [slots]: every sequence's last token of the step before; updated to this step's."""
+    _gpu(resid, table, last)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    if table.dim() != 2 or tuple(table.shape) != (buckets + 1, H) or not table.is_contiguous():
+        raise KernelError(f"pair_embed: the table must be contiguous [{buckets + 1}, {H}]")
+    if last.dtype != torch.int32 or not last.is_contiguous():
+        raise KernelError("pair_embed: the last tokens are contiguous int32, one a state slot")
+    B = ctx.num_seqs
+    _i32(ctx.token_ids, "token_ids", T); _i32(ctx.positions, "positions", T); _i32(ctx.token_seq, "token_seq", T)
+    _i32(ctx.cu_seqlens, "cu_seqlens", B + 1); _i32(ctx.state_slots, "state_slots", B)
+    lib = library.core()
+    _check(lib, lib.pico_pair_embed(_ptr(resid), _ptr(table), _dt(table), _ptr(ctx.token_ids), _ptr(ctx.positions),
+                                    _ptr(ctx.token_seq), _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(last), last.numel(),
+                                    c_ll(mul_prev), c_ll(mul_cur), buckets, T, B, H, _stream()))
+    return resid
+
+
+# ---- attention through latents ---------------------------------------------------------------------------------------
+def latent_prepare(y: torch.Tensor, q_rank: int, kv_rank: int, rot: int, wq: torch.Tensor, wkv: torch.Tensor, eps: float,
+                   cos_sin: Optional[torch.Tensor], slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+    """y [T, q_rank + kv_rank + rot]: returns the normed query latent [T, q_rank]; writes the normed key/value latent and
+    the turned rotated key part into the cache (K rows [latent | rotated part], V columns the latent again)."""
+    _gpu(y, wq, wkv, cos_sin, slots, k_cache, v_cache)
+    T = y.shape[0]
+    if y.dim() != 2 or y.stride(1) != 1 or y.shape[1] < q_rank + kv_rank + rot:
+        raise KernelError("latent_prepare: the rows do not hold the two latents and the rotated part")
+    pages, P = _check_cache2(k_cache, v_cache, 1, kv_rank + rot, kv_rank)
+    if k_cache.dtype != y.dtype:
+        raise KernelError("cache and activations differ in dtype")
+    _vec(wq, q_rank, "the query latent's norm weight"); _vec(wkv, kv_rank, "the key/value latent's norm weight")
+    _i32(slots, "slots", T)
+    if rot:
+        _check_table(cos_sin, T, rot // 2)
+    cq = torch.empty(T, q_rank, dtype=y.dtype, device=y.device)
+    lib = library.core()
+    _check(lib, lib.pico_latent_prepare(_ptr(y), y.stride(0) if T > 1 else y.shape[1], _dt(y), q_rank, kv_rank, rot, _ptr(wq),
+                                        _ptr(wkv), c_float(eps), _ptr(cos_sin), _ptr(slots), _ptr(cq), _ptr(k_cache),
+                                        _ptr(v_cache), T, P, pages, _stream()))
+    return cq
+
+
+def rope_inplace(x: torch.Tensor, col0: int, heads: int, head_stride: int, rot: int, cos_sin: torch.Tensor, halves: bool) -> torch.Tensor:
+    """Turn ``rot`` entries from column col0 + h * head_stride of every row of x, for h < heads, by the angles of
+    ``cos_sin`` (``rope_table``): neighbouring pairs, or with ``halves`` entry i with entry i + rot / 2."""
+    _gpu(x, cos_sin)
+    T = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("rope_inplace: x must be [T, columns] with unit stride along the row")
+    if rot:
+        _check_table(cos_sin, T, rot // 2)
+    lib = library.core()
+    _check(lib, lib.pico_rope_inplace(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), col0, heads, head_stride, rot,
+                                      1 if halves else 0, _ptr(cos_sin), T, _stream()))
+    return x
+
+
+def head_linear(x: torch.Tensor, x_col: int, x_head: int, w: torch.Tensor, heads: int, copy: int = 0,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A product a head: out[t, h, :n_out] = x[t, x_col + h * x_head : .. + n_in] @ w[h] with w [heads, n_in, n_out];
+    the ``copy`` entries behind a head's inputs are handed on behind its outputs.  Returns [T, heads * (n_out + copy)]."""
+    _gpu(x, w, out)
+    T = x.shape[0]
+    if w.dim() != 3 or w.shape[0] != heads or not w.is_contiguous() or w.dtype != x.dtype:
+        raise KernelError("head_linear: w must be contiguous [heads, in, out] of the activations' dtype")
+    n_in, n_out = w.shape[1], w.shape[2]
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("head_linear: x must be [T, columns] with unit stride along the row")
+    o_head = n_out + copy
+    if out is None:
+        out = torch.empty(T, heads * o_head, dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != (T, heads * o_head) or out.dtype != x.dtype or not out.is_contiguous():
+        raise KernelError("head_linear: out has the wrong shape or dtype")
+    lib = library.core()
+    _check(lib, lib.pico_head_linear(_ptr(x), x.stride(0) if T > 1 else x.shape[1], x_col, x_head, _ptr(w), _ptr(out),
+                                     heads * o_head, 0, o_head, _dt(x), T, heads, n_in, n_out, copy, _stream()))
+    return out
+
+
+# ---- the selective state-space mixer -----------------------------------------------------------------------------------
+SSM_MAX_TAPS, SSM_MAX_STATE = 16, 256
+
+
+def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Tensor, ctx, state: torch.Tensor, n_state: int) -> torch.Tensor:
+    """silu(bias + the causal convolution of the first ``channels`` columns of x with w [channels, taps]) for every
+    sequence of the step; inputs before a portion come from the slot's history (``state`` float32
+    [slots, channels, n_state + taps - 1], its last taps - 1 columns), which is brought up to date."""
+    _gpu(x, w, bias, state)
+    T = x.shape[0]
+    taps = w.shape[1]
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < channels:
+        raise KernelError("causal_conv: the rows do not hold the channels")
+    if w.dtype != torch.float32 or tuple(w.shape) != (channels, taps) or not w.is_contiguous() or not 1 <= taps <= SSM_MAX_TAPS:
+        raise KernelError(f"causal_conv: the taps are contiguous float32 [{channels}, 1 to {SSM_MAX_TAPS}]")
+    _vec(bias, channels, "the convolution's bias")
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (channels, n_state + taps - 1) or not state.is_contiguous():
+        raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {channels}, {n_state + taps - 1}]")
+    B = ctx.num_seqs
+    _i32(ctx.token_seq, "token_seq", T); _i32(ctx.cu_seqlens, "cu_seqlens", B + 1); _i32(ctx.state_slots, "state_slots", B)
+    out = torch.empty(T, channels, dtype=x.dtype, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_causal_conv(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), _ptr(w), _ptr(bias), _ptr(ctx.token_seq),
+                                     _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(state), state.shape[0], T, B, channels,
+                                     n_state, taps, _ptr(out), _stream()))
+    return out
+
+
+def selective_scan(xc: torch.Tensor, dt_pre: torch.Tensor, dt_bias: torch.Tensor, bc: torch.Tensor, b_col: int, c_col: int,
+                   a_log: torch.Tensor, d: torch.Tensor, z: torch.Tensor, ctx, state: torch.Tensor, hist: int) -> torch.Tensor:
+    """The recurrence S <- exp(dt A) S + dt x B, y = S . C + D x with dt = softplus(dt_pre + dt_bias), A = -exp(a_log), for
+    every sequence of the step from its state slot (``state`` float32 [slots, channels, N + hist], updated in place);
+    returns y * silu(z) [T, channels] in xc's dtype.  xc [T, channels]; dt_pre float32 [T, channels]; B and C are
+    columns b_col .. and c_col .. of ``bc``; z [T, >= channels] (row stride free)."""
+    _gpu(xc, dt_pre, dt_bias, bc, a_log, d, z, state)
+    T, C = xc.shape
+    N = a_log.shape[1]
+    if not xc.is_contiguous() or dt_pre.dtype != torch.float32 or tuple(dt_pre.shape) != (T, C) or not dt_pre.is_contiguous():
+        raise KernelError("selective_scan: xc [T, channels] contiguous and dt_pre float32 of the same shape")
+    if a_log.dtype != torch.float32 or tuple(a_log.shape) != (C, N) or not a_log.is_contiguous() or N > SSM_MAX_STATE:
+        raise KernelError(f"selective_scan: a_log must be contiguous float32 [{C}, at most {SSM_MAX_STATE}]")
+    _vec(dt_bias, C, "dt bias"); _vec(d, C, "D")
+    if bc.dtype != xc.dtype or bc.dim() != 2 or bc.shape[0] != T or bc.stride(1) != 1 or bc.shape[1] < max(b_col, c_col) + N:
+        raise KernelError("selective_scan: the rows of bc do not hold B and C")
+    if z.dtype != xc.dtype or z.dim() != 2 or z.shape[0] != T or z.stride(1) != 1 or z.shape[1] < C:
+        raise KernelError("selective_scan: z must be [T, >= channels] of the activations' dtype")
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (C, N + hist) or not state.is_contiguous():
+        raise KernelError(f"selective_scan: the state must be contiguous float32 [slots, {C}, {N + hist}]")
+    B = ctx.num_seqs
+    _i32(ctx.cu_seqlens, "cu_seqlens", B + 1); _i32(ctx.state_slots, "state_slots", B)
+    out = torch.empty(T, C, dtype=xc.dtype, device=xc.device)
+    lib = library.core()
+    _check(lib, lib.pico_selective_scan(_ptr(xc), _ptr(dt_pre), _ptr(dt_bias), _ptr(bc), bc.stride(0) if T > 1 else bc.shape[1],
+                                        b_col, c_col, _ptr(a_log), _ptr(d), _ptr(z), z.stride(0) if T > 1 else z.shape[1], _dt(xc),
+                                        _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(state), state.shape[0], B, T, C, N, hist,
+                                        _ptr(out), _stream()))
+    return out
+
+
+def moe_router_top_softmax(x: torch.Tensor, w_router: torch.Tensor, bias: Optional[torch.Tensor], experts: int, top: int):
+    """Router logits z = x w_router^T (+ bias on the first ``experts`` of them) in float32; the ``top`` largest of the
+    experts' logits are chosen (the lowest index among equals), weights = softmax over the chosen logits.  Rows of
+    w_router behind the experts' give further logits that take no part (returned with the others).
+    Returns (experts int32 [T, top], weights float32 [T, top], z float32 [T, rows of w_router])."""
+    _gpu(x, w_router, bias)
+    T, D = x.shape
+    rows = w_router.shape[0]
+    if w_router.dtype != torch.float32 or w_router.dim() != 2 or w_router.shape[1] != D or not w_router.is_contiguous() or rows < experts:
+        raise KernelError(f"moe_router_top_softmax: the router matrix must be contiguous float32 [>= {experts}, {D}]")
+    _vec(bias, experts, "the router's bias")
+    if x.stride(1) != 1:
+        raise KernelError("moe_router_top_softmax: activations must have unit stride along the row")
+    if not 1 <= top <= min(experts, MOE_MAX_TOP):
+        raise KernelError(f"moe_router_top_softmax: {top} of {experts} experts per token (at most {MOE_MAX_TOP})")
+    z = torch.empty(T, rows, dtype=torch.float32, device=x.device)
+    chosen = torch.empty(T, top, dtype=torch.int32, device=x.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_moe_router_top_softmax(_ptr(x), x.stride(0) if T > 1 else D, _dt(x), _ptr(w_router), _ptr(bias), T,
+                                                experts, rows - experts, D, top, _ptr(z), _ptr(chosen), _ptr(weights), _stream()))
+    return chosen, weights, z

@@ -168,6 +168,11 @@ class StreamPart(Part):
     """A part that works on the residual stream outside the layers (``ModelSpec.before_layers`` /
     ``after_layers``): learned absolute positions added to the embeddings, a norm of the embeddings."""
 
+    def cache_spec(self) -> CacheSpec:
+        """What the part keeps per request between steps: nothing, or a state of fixed size (a token seen in the step
+        before, say).  A part with state is called as ``forward(resid, ctx, cache)`` with its ``StateLayer``."""
+        return CacheSpec("none")
+
     def forward(self, resid: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
         """resid: float32 [T, H], the residual stream (with nothing pending); returns it (changed in place or anew)."""
         raise NotImplementedError
@@ -217,6 +222,13 @@ class Block(Part):
 
     def __init__(self, parts: Dict[str, Part]):
         self.parts = parts
+
+    def own_param_specs(self) -> List[ParamSpec]:
+        """Tensors of the arrangement itself (named behind the layer's prefix), beside those of its parts."""
+        return []
+
+    def load_own(self, tensors: Dict[str, torch.Tensor], device: torch.device, dtype: torch.dtype) -> None:
+        pass
 
     def _sub_parts(self) -> List[Part]:
         return list(self.parts.values())

@@ -107,3 +107,67 @@ class ParallelTwoNormBlock(Block):
                 self._add(resid, d)
             f = f[-1]
         return resid, f
+
+
+@register_part("block", "prenorm_scaled")
+class ScaledPreNormBlock(Block):
+    """x += m * s1 * mixer(norm1(x));  x += m * s2 * ff(norm2(x)): the pre-norm arrangement with a constant ``mult`` and
+    a stored vector a sublayer (``scale_names``, behind the layer's prefix) on what joins the residual stream.  The
+    products m * s are made once at load; the sums are float32.  The mixer's scaled output joins the stream in the
+    launch of norm2 where that norm takes a scale on its addend (``takes_delta_scale``); the feed-forward's joins at
+    once (a feed-forward with ``forward_scaled_into(h, ctx, resid, scale)`` adds it itself, in the launch that puts its
+    pieces together), so nothing is handed on as pending.  A layer without a feed-forward names the part "none"."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ff": "feed_forward"}
+    graph_safe_prompts = True
+
+    def __init__(self, parts, size: int, mult: float = 1.0, scale_names=("ls1", "ls2")):
+        super().__init__(parts)
+        self.size, self.mult, self.scale_names = int(size), float(mult), tuple(scale_names)
+        self.s1 = self.s2 = None
+
+    def own_param_specs(self):
+        from .spec import ParamSpec
+        return [ParamSpec(n, (self.size,), role="norm") for n in self.scale_names]
+
+    def load_own(self, tensors, device, dtype) -> None:
+        import torch
+        self.s1, self.s2 = ((tensors[n].to(device=device, dtype=torch.float32) * self.mult).contiguous() for n in self.scale_names)
+
+    def forward(self, resid, pending, ctx, cache):
+        p = self.parts
+        h = p["norm1"].add_norm(resid, pending)
+        a = p["mixer"].forward(h, ctx, cache)
+        if getattr(p["norm2"], "takes_delta_scale", False) and not (a.dim() == 3 and a.shape[0] > kernels.LN_MAX_SLABS):
+            h = p["norm2"].add_norm(resid, a, delta_scale=self.s1)
+        else:
+            kernels.scaled_add(resid, a, scale=self.s1)
+            h = p["norm2"].add_norm(resid, None)
+        into = getattr(p["ff"], "forward_scaled_into", None)
+        if into is not None:
+            into(h, ctx, resid, self.s2)
+            return resid, None
+        f = p["ff"].forward(h, ctx)
+        for d in (f if isinstance(f, (list, tuple)) else (f,)):
+            if d is not None:
+                kernels.scaled_add(resid, d, scale=self.s2)
+        return resid, None
+
+
+@register_part("block", "prenorm_scaled_mixer_only")
+class ScaledMixerOnlyBlock(ScaledPreNormBlock):
+    """x += m * s1 * mixer(norm1(x)) and nothing else: the arrangement above for a layer without a feed-forward (and so
+    without a second norm and a second vector)."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer"}
+
+    def __init__(self, parts, size: int, mult: float = 1.0, scale_names=("ls1",)):
+        super().__init__(parts, size, mult, tuple(scale_names)[:1])
+
+    def load_own(self, tensors, device, dtype) -> None:
+        import torch
+        self.s1 = (tensors[self.scale_names[0]].to(device=device, dtype=torch.float32) * self.mult).contiguous()
+
+    def forward(self, resid, pending, ctx, cache):
+        p = self.parts
+        h = p["norm1"].add_norm(resid, pending)
+        kernels.scaled_add(resid, p["mixer"].forward(h, ctx, cache), scale=self.s1)
+        return resid, None

@@ -9,7 +9,7 @@ from ..config.registry import load_model_description
 from ..ops import kernels
 from ..ops.linear import Linear
 from ..weights.loader import load_checkpoint
-from . import attention, attention_bias, attention_gated, block, gla, mlp, moe, norm, positions, rotary  # noqa: F401  (register the parts)
+from . import attention, attention_bias, attention_gated, block, gla, latent_attention, mlp, moe, norm, positions, retention, rotary, ssm  # noqa: F401  (register the parts)
 from .base import Block, StepContext
 from .registry import build_part, part_class
 from .spec import CacheSpec, ModelSpec, ParamSpec
@@ -33,7 +33,7 @@ def _build_layer(lspec, act_dtype) -> Tuple[Block, Dict[str, str]]:
         name, pspec = lspec.slots[slot]
         parts[slot] = build_part(cat, pspec, act_dtype=act_dtype)
         sub[slot] = name
-    return cls(parts), sub
+    return cls(parts, **lspec.block_params), sub
 
 
 def _layer_params(lspec, blk: Block, sub: Dict[str, str]) -> List[Tuple[str, str, ParamSpec]]:
@@ -43,6 +43,9 @@ def _layer_params(lspec, blk: Block, sub: Dict[str, str]) -> List[Tuple[str, str
         for p in part.param_specs():
             full = tensor_name(lspec.prefix, sub[slot], p.name)
             out.append((slot, full, ParamSpec(full, p.shape, p.role, p.std)))
+    for p in blk.own_param_specs():
+        full = tensor_name(lspec.prefix, p.name)
+        out.append(("", full, ParamSpec(full, p.shape, p.role, p.std)))
     return out
 
 
@@ -97,8 +100,22 @@ class DecoderModel:
                     raise ValueError(f"run entry {i} cannot use the cache of entry {e.cache_of}: different cache needs")
 
     def cache_specs(self) -> Dict[int, CacheSpec]:
-        """CacheSpec by cache id (the index of the run entry that owns the cache)."""
-        return {i: self.layers[self.spec.run_order[i].layer].mixer.cache_spec() for i in self.spec.cache_owners()}
+        """CacheSpec by cache id: the index of the run entry that owns the cache; -(k + 1) for the k-th part around the
+        layers (``before_layers``, then ``after_layers``) that keeps a state."""
+        out = {i: self.layers[self.spec.run_order[i].layer].mixer.cache_spec() for i in self.spec.cache_owners()}
+        for k, (_, part) in enumerate(self.before + self.after):
+            cs = part.cache_spec()
+            if cs.kind == "state":
+                out[-(k + 1)] = cs
+            elif cs.kind != "none":
+                raise ValueError("a part around the layers keeps a state of fixed size or nothing")
+        return out
+
+    def _run_stream(self, k: int, part, resid, ctx, storage):
+        """Part k of those around the layers, with its state if it keeps one."""
+        if part.cache_spec().kind == "state":
+            return part.forward(resid, ctx, storage.layer(-(k + 1)))
+        return part.forward(resid, ctx)
 
     def param_specs(self) -> List[ParamSpec]:
         return model_param_specs(self.spec)
@@ -110,6 +127,7 @@ class DecoderModel:
             for slot, part in blk.parts.items():
                 part.load({p.name: tensors[tensor_name(lspec.prefix, sub[slot], p.name)] for p in part.param_specs()},
                           dev, self.dtype)
+            blk.load_own({p.name: tensors[tensor_name(lspec.prefix, p.name)] for p in blk.own_param_specs()}, dev, self.dtype)
         for prefix, part in self.before + self.after:
             part.load({p.name: tensors[tensor_name(prefix, p.name)] for p in part.param_specs()}, dev, self.dtype)
         self.final_norm.load({p.name: tensors[tensor_name(spec.final_norm_name, p.name)]
@@ -157,10 +175,14 @@ class DecoderModel:
     def _forward(self, ctx: StepContext, storage) -> torch.Tensor:
         ctx.shared.clear()      # what layers share belongs to this pass (a context may be run again, as at graph capture)
         resid = kernels.embedding(self.embed, ctx.token_ids[:ctx.num_tokens], scale=self.spec.embed_scale)
-        for _, part in self.before:
-            resid = part.forward(resid, ctx)
+        for k, (_, part) in enumerate(self.before):
+            resid = self._run_stream(k, part, resid, ctx, storage)
+        # runs that take the layers' input again: a copy of the stream as it is now
+        entered = resid.clone() if any(e.add_input for e in self.spec.run_order) else None
         pending = None
         for i, e in enumerate(self.spec.run_order):
+            if e.add_input:
+                kernels.residual_add(resid, entered)       # what is pending joins later; the sums are float32
             # a run that names another run's cache reads it and stores nothing of its own
             resid, pending = self.layers[e.layer].forward(resid, pending, ctx,
                                                           storage.layer(self.spec.cache_id(i), read_only=e.cache_of is not None))
@@ -171,8 +193,8 @@ class DecoderModel:
                 for delta in (pending if pending.dim() == 3 else (pending,)):       # a stack of partial sums: each in turn
                     kernels.residual_add(resid, delta)
                 pending = None
-            for _, part in self.after:
-                resid = part.forward(resid, ctx)
+            for k, (_, part) in enumerate(self.after):
+                resid = self._run_stream(len(self.before) + k, part, resid, ctx, storage)
         h = self.final_norm.add_norm(resid, pending, rows=ctx.want_rows)
         logits = self.head(h, out_dtype=torch.float32)
         if self.spec.logit_softcap > 0:

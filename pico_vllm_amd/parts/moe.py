@@ -189,3 +189,69 @@ class SoftmaxRoutedExperts(FeedForward):
 
     def graph_variant(self, ctx: StepContext) -> tuple:
         return (("softmax_routed_experts", kernels.moe_grouped_rows(ctx.num_tokens, self.top)),)
+
+
+@register_part("feed_forward", "top_softmax_routed_experts")
+class TopSoftmaxRoutedExperts(SoftmaxRoutedExperts):
+    """Router: z = x Wr^T + b in float32; the ``top`` experts with the largest logits are chosen (the lowest index among
+    equals), and their weights are the softmax over the chosen logits only.  Experts as in ``SoftmaxRoutedExperts``
+    (Wd_e (silu(Wg_e x) * (Wu_e x)), the weight on the output).  With ``shared_size`` > 0 one more gated feed-forward
+    runs for every token; with ``shared_gate_name`` its output is multiplied by sigmoid(wsg . x), one number a token
+    (the gate's row rides behind the router's rows: one launch makes the experts' logits and the gate's).
+
+    ``forward_scaled_into(x, ctx, resid, scale)`` adds scale * (routed sum + gated shared output) to the float32 stream
+    in the one launch that puts the pieces together."""
+
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, shared_size: int = 0,
+                 router_name: str = "router", router_bias_name: Optional[str] = "router.b",
+                 shared_gate_name: Optional[str] = "shared.sg", expert_names: tuple = ("e{}.gate", "e{}.up", "e{}.down"),
+                 shared_names: tuple = ("shared.gate", "shared.up", "shared.down"), act_dtype: torch.dtype = torch.bfloat16):
+        super().__init__(hidden_size, expert_size, num_experts, top, identity=0, scale=1.0, shared_size=shared_size,
+                         correction_name=None, router_name=router_name, expert_names=expert_names, shared_names=shared_names,
+                         act_dtype=act_dtype)
+        self.router_bias_name = router_bias_name
+        self.shared_gate_name = shared_gate_name if shared_size else None
+        self.router_bias: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        out = super().param_specs()
+        if self.router_bias_name:
+            out.append(ParamSpec(self.router_bias_name, (self.num_experts,), role="f32"))
+        if self.shared_gate_name:
+            out.append(ParamSpec(self.shared_gate_name, (1, self.hidden_size)))
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        super().load(tensors, device, dtype)
+        if self.shared_gate_name:       # the gate's row behind the experts' rows, float32 like them
+            self.router = Linear(torch.cat([self.router.weight, tensors[self.shared_gate_name].float().to(device)], dim=0))
+        if self.router_bias_name:
+            self.router_bias = tensors[self.router_bias_name].to(device=device, dtype=torch.float32).contiguous()
+
+    def _pieces(self, x: torch.Tensor, ctx: StepContext):
+        """(routed sum, shared expert's output or None, its gate's logits or None)."""
+        E, F, D = self.num_experts, self.expert_size, self.hidden_size
+        experts, weights, z = kernels.moe_router_top_softmax(x, self.router.weight, self.router_bias, E, self.top)
+        gate_up = self.gate_up.weight.view(E, 2 * F, D)
+        down = self.down.weight.view(E, D, F)
+        xe = x if x.dtype == gate_up.dtype else x.to(gate_up.dtype)
+        if kernels.moe_fast_ok(xe, gate_up, down):
+            routed = kernels.moe_experts(xe, gate_up, down, experts, weights, 0.0, 0.0, mode=kernels.MOE_SWIGLU)
+        else:
+            routed = kernels.moe_experts_plain(xe, gate_up, down, experts, weights, 0.0, 0.0, mode=kernels.MOE_SWIGLU)
+        if self.shared is None:
+            return routed, None, None
+        shared = self.shared.down(self.shared.gate_up.swiglu(x))          # [T, D], one piece: the gate multiplies it
+        return routed, shared, (z[:, E:] if self.shared_gate_name else None)
+
+    def forward_scaled_into(self, x: torch.Tensor, ctx: StepContext, resid: torch.Tensor, scale: Optional[torch.Tensor]) -> None:
+        routed, shared, gate = self._pieces(x, ctx)
+        kernels.scaled_add(resid, routed, shared, gate, scale)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext):
+        routed, shared, gate = self._pieces(x, ctx)
+        out = torch.zeros(x.shape[0], self.hidden_size, dtype=torch.float32, device=x.device)
+        kernels.scaled_add(out, routed, shared, gate, None)
+        return out
+
+    forward_into = None        # the parent's way of adding the shared expert knows no gate

@@ -42,3 +42,30 @@ class RMSNorm(Norm):
                 and (delta is None or delta.dtype == torch.float32)):
             return DeferredNorm(self, resid, delta, "rms", self.weight, self.eps)
         return None
+
+
+@register_part("norm", "layer_norm")
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean squared deviation, in float32.  The sum in front
+    of it may be scaled element by element: ``add_norm(resid, delta, delta_scale=s)`` norms resid + s * delta."""
+    graph_safe_prompts = True
+    takes_delta_scale = True
+
+    def __init__(self, size: int, eps: float, act_dtype: torch.dtype = torch.bfloat16, weight_name: str = "weight",
+                 bias_name: str = "bias"):
+        self.size, self.eps, self.act_dtype = size, eps, act_dtype
+        self.weight_name, self.bias_name = weight_name, bias_name
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        return [ParamSpec(self.weight_name, (self.size,), role="norm"), ParamSpec(self.bias_name, (self.size,), role="f32")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        self.weight = tensors[self.weight_name].to(device=device, dtype=torch.float32).contiguous()
+        self.bias = tensors[self.bias_name].to(device=device, dtype=torch.float32).contiguous()
+
+    def add_norm(self, resid, delta, rows=None, delta_scale=None):
+        if delta is not None and delta.dim() == 3 and delta.shape[0] > kernels.LN_MAX_SLABS:
+            raise ValueError(f"a layer norm's launch adds at most {kernels.LN_MAX_SLABS} partial sums")
+        return kernels.add_layernorm(resid, delta, self.weight, self.bias, self.eps, self.act_dtype, rows, delta_scale)

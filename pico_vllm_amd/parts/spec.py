@@ -26,6 +26,7 @@ class ParamSpec:
       matrix  - bfloat16 (float32 in the 32-bit engine, or if stored in 32 bit); N(0, std)
       bias    - like matrix; N(0, std)
       norm    - float32 always; 1 + U(-0.1, 0.1)
+      f32     - float32 always (a norm's bias, what enters a recurrence); N(0, std)
       table   - int32 integer table; zeros
     """
     name: str
@@ -91,6 +92,9 @@ class LayerSpec:
     prefix: str
     block: str
     slots: Dict[str, Tuple[str, PartSpec]]
+    # constants of the arrangement itself (a multiplier on what joins the residual stream, say); an arrangement may
+    # also own tensors, named behind the layer's prefix (``Block.own_param_specs``)
+    block_params: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -98,9 +102,12 @@ class RunEntry:
     """One entry of the run order: run ``layer`` (an index into ``layers``; a
     layer may be named by several entries, which then share its weights).
     Every entry owns a cache of its own unless ``cache_of`` names an EARLIER
-    entry of the run order, whose cache this run's mixer is then given."""
+    entry of the run order, whose cache this run's mixer is then given.
+    ``add_input``: the residual stream as it entered the first layer (the embeddings with everything
+    ``before_layers`` did to them) is added to the stream in front of this run."""
     layer: int
     cache_of: Optional[int] = None
+    add_input: bool = False
 
 
 @dataclass(frozen=True)

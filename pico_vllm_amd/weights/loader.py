@@ -44,7 +44,7 @@ class WeightsError(ValueError):
 def kept_dtype(role: str, stored: torch.dtype, engine_dtype: torch.dtype) -> torch.dtype:
     if role == "table":
         return torch.int32
-    if role == "norm" or engine_dtype == torch.float32:
+    if role in ("norm", "f32") or engine_dtype == torch.float32:
         return torch.float32
     if stored in (torch.float32, torch.float64):
         return torch.float32          # stored in 32 bit: stays so
