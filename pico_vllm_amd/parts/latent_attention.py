@@ -101,7 +101,8 @@ class LatentAttention(Mixer):
             self.position.load({}, device, dtype)
         if self.act_dtype == torch.bfloat16 and self.uk_t.dtype == torch.bfloat16:
             from ..ops import attention_bias_fast
-            if attention_bias_fast.supported(self.dk, self.kv_rank):
+            # (the matrix-core kernel reads query rows in 16-byte pieces)
+            if attention_bias_fast.supported(self.dk, self.kv_rank) and (self.heads * self.dk) % 8 == 0:
                 self.fast = attention_bias_fast.FastBiasAttention(self.nq, 1, self.dk, self.kv_rank, self.scale)
 
     def graph_variant(self, ctx: StepContext) -> tuple:

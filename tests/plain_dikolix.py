@@ -167,7 +167,8 @@ def retention_recurrence(q, k, v, decay, state=None):
     return torch.stack(out), S
 
 
-def retention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float, positions: torch.Tensor) -> torch.Tensor:
+def retention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float, positions: torch.Tensor,
+              margins_out: Optional[List] = None) -> torch.Tensor:
     n = h.shape[0]
     H, dk, dv = m["heads"], m["dim"], m["vdim"]
     q = (h @ w["q"].T).view(n, H, dk)
@@ -177,6 +178,11 @@ def retention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float, 
         q, k = rotate(q, positions, m["rot"], "halves"), rotate(k, positions, m["rot"], "halves")
     k = k * dk ** -0.5
     o, _ = retention_recurrence(q, k, v, torch.tensor(m["decay"], dtype=h.dtype))
+    if margins_out is not None:
+        # where a head's output cancels to a small part of what went into it, a rounding decides its direction and the
+        # norm behind it blows that up: 4 |o| / (|q| * the largest |k| |v| so far), the least over the heads
+        kv = torch.cummax(k.norm(dim=-1) * v.norm(dim=-1), 0).values
+        margins_out.append((4.0 * o.norm(dim=-1) / (q.norm(dim=-1) * kv + 1e-300)).min(-1).values)
     o = rms_norm(o, None, eps).reshape(n, H * dv)
     return (o * silu(h @ w["g"].T)) @ w["o"].T
 
@@ -195,9 +201,20 @@ def route(h: torch.Tensor, router: torch.Tensor, bias: torch.Tensor, top: int):
     return idx, torch.softmax(val, dim=-1), z
 
 
-def moe(h: torch.Tensor, w: Dict[str, torch.Tensor], f: dict) -> torch.Tensor:
+def route_margin(z: torch.Tensor, top: int) -> torch.Tensor:
+    """Per token: how far the last chosen logit lies above the first rejected one, in units of the row's spread
+    (infinite where every expert is chosen).  A small margin means that a rounding may choose otherwise."""
+    if top >= z.shape[-1]:
+        return torch.full((z.shape[0],), float("inf"), dtype=z.dtype)
+    val, _ = torch.topk(z, top + 1, dim=-1)
+    return (val[:, top - 1] - val[:, top]) / (z.std(-1) + 1e-12)
+
+
+def moe(h: torch.Tensor, w: Dict[str, torch.Tensor], f: dict, margins_out: Optional[List] = None) -> torch.Tensor:
     E, top = f["router"]["experts"], f["router"]["top"]
-    idx, wt, _ = route(h, w["router"], w["router.b"], top)
+    idx, wt, z = route(h, w["router"], w["router.b"], top)
+    if margins_out is not None:
+        margins_out.append(route_margin(z, top))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(top):
@@ -228,8 +245,10 @@ def run_order(config: dict) -> List[tuple]:
     return out + [(i, False) for i in range(loop["stop"], n)]
 
 
-def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None) -> torch.Tensor:
-    """Logits [n, vocab] of one whole sequence."""
+def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.float64, layers_out: Optional[List] = None,
+            margins_out: Optional[List] = None) -> torch.Tensor:
+    """Logits [n, vocab] of one whole sequence.  ``layers_out`` gets the residual stream after every layer run,
+    ``margins_out`` every routed layer run's margins of the choice (``route_margin``)."""
     tokens = [int(t) for t in tokens]
     eps, mult = config["norm"]["eps"], config.get("residual_mult", 1.0)
     pos = torch.arange(len(tokens))
@@ -247,14 +266,14 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens, dtype=torch.
         elif l["type"] == "mamba1":
             a = mamba(h, mw, l["mixer"])
         elif l["type"] == "retention":
-            a = retention(h, mw, l["mixer"], eps, pos)
+            a = retention(h, mw, l["mixer"], eps, pos, margins_out)
         else:
             raise ValueError(l["type"])
         x = x + mult * w["ls1"] * a
         if l.get("mlp"):
             h = layer_norm(x, w["norm2"], w["norm2.b"], eps)
             fw = {k[4:]: v for k, v in w.items() if k.startswith("mlp.")}
-            x = x + mult * w["ls2"] * moe(h, fw, l["mlp"])
+            x = x + mult * w["ls2"] * moe(h, fw, l["mlp"], margins_out)
         if layers_out is not None:
             layers_out.append(x.clone())
     h = layer_norm(x, tensors["final.norm"].to(dtype), tensors["final.norm.b"].to(dtype), eps)
