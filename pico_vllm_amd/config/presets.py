@@ -79,6 +79,33 @@ DESIGN_PRESETS.update({
 })
 
 
+def _dikolix(vocab, width, layers, heads, dim, rot_dim, q_rank, kv_rank, experts, top, expert_ff, shared_ff, ret_dim=64,
+             buckets=262144) -> Dict:
+    """A Dikolix configuration of a real model's proportions, in groups of three layers: attention through latents, a
+    selective state-space layer of twice the width, retention; every layer with routed experts and a gated shared one;
+    a hashed table of token pairs on the embedding."""
+    att = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": dim, "q_rank": q_rank, "kv_rank": kv_rank,
+           "scale": (dim + rot_dim) ** -0.5,
+           "rot": {"dims": rot_dim, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 8192, "fast": 16.0, "slow": 2.0}}}
+    ssm = {"inner": 2 * width, "state": 16, "conv": 4, "dt_rank": width // 16}
+    ret = {"heads": heads, "dim": ret_dim, "vdim": dim, "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * h / heads) for h in range(heads)],
+           "rot": {"dims": ret_dim, "base": 10000.0}}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": shared_ff}}
+    kinds = (("latent_attention", att), ("mamba1", ssm), ("retention", ret))
+    return {"architecture": "Dikolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.8,
+            "embedding": {"bigram": {"buckets": buckets, "mul_prev": 1000003, "mul_cur": 31}},
+            "layers": [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": routed} for i in range(layers)]}
+
+
+# Dikolix at the sizes of the Qwen2.5 shapes: the same width, heads and head size; the routed feed-forward of the Nasedra
+# presets in every layer; a key/value latent of 256 entries and a rotated part of 64 (the largest value size the
+# matrix-core attention of this package takes is 256).
+DESIGN_PRESETS.update({
+    "dikolix-1.5b": _dikolix(151936, 1536, 27, 12, 128, 64, 768, 256, 16, 2, 2240, 4480),
+    "dikolix-7b": _dikolix(152064, 3584, 27, 28, 128, 64, 1536, 256, 32, 4, 2368, 9472),
+})
+
+
 def preset(name: str) -> Dict:
     import copy
     key = name.lower()

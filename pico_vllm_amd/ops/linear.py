@@ -69,6 +69,21 @@ def _library_tuning(rows: int) -> None:
         st["tuning"] = want
 
 
+class no_library_tuning:
+    """Inside the scope the library's tuner times nothing (a product it has no tuned result for takes the library's
+    default choice); afterwards the next ``Linear`` call sets the mode it wants as before."""
+
+    def __enter__(self):
+        st = _tuner_state
+        if st["ready"] is True and st["tuning"]:
+            torch.cuda.tunable.tuning_enable(False)
+            st["tuning"] = False
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
 class Linear:
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
         if weight.dim() != 2:

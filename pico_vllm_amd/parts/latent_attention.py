@@ -112,10 +112,17 @@ class LatentAttention(Mixer):
         """out[t, h] = [x[t, h, :in] @ w[h] | x[t, h, in : in + copy]]; x [T, H * x_head]."""
         T, H = x.shape[0], self.heads
         if x.dtype == torch.bfloat16 and T >= self.LIBRARY_FROM:
+            # The library's batched product on operands laid out batch by batch ([H, T, in] and [H, T, out], both made
+            # here), and never under the library's tuner: handed the rows' own layout (a head's matrix interleaved
+            # with the other heads', the batch stride smaller than the row stride) the tuner's copies of the operands
+            # are sized for batch-major ones and it reads beyond them.
+            from ..ops.linear import no_library_tuning
             n_in, n_out = w.shape[1], w.shape[2]
             xv = x.view(T, H, x_head)
             out = torch.empty(T, H, n_out + copy, dtype=x.dtype, device=x.device)
-            out[:, :, :n_out] = torch.bmm(xv[:, :, :n_in].transpose(0, 1), w).transpose(0, 1)
+            with no_library_tuning():
+                res = torch.bmm(xv[:, :, :n_in].transpose(0, 1).contiguous(), w)          # [H, T, out]
+            out[:, :, :n_out] = res.transpose(0, 1)
             if copy:
                 out[:, :, n_out:] = xv[:, :, n_in:n_in + copy]
             return out.view(T, H * (n_out + copy))
