@@ -80,13 +80,24 @@ extern "C" int pico_causal_conv(const void* x, int ldx, int dtype, const float* 
 }
 
 // ---------------------------------------------------------------------------
-// The recurrence.  grid (sequences, ceil(C / channels a workgroup)); LPC lanes (a power of two, at most 64) share a
-// channel, lane l of them owns state elements l, l + LPC, .. (NPL of them); the sum over n is a lane's chain and then
-// a butterfly over the LPC lanes.  Tokens are taken SSM_TB at a time so that their loads travel together.
+// The recurrence.  grid (sequences, ceil(C / channels a workgroup)); LPC lanes (a power of two: 1 up to 16 state
+// elements, so that a lane owns at most 16) share a channel, lane l of them owns state elements l, l + LPC, .. (NPL of
+// them); the sum over n is a lane's chain and then a butterfly over the LPC lanes.  Tokens are taken SSM_TB at a time:
+// a thread's own values (its channel's input, step size and gate: neighbouring threads read neighbouring channels)
+// travel together in registers, and the tokens' B and C rows, which all channels share, are staged in LDS.
 // ---------------------------------------------------------------------------
-#define SSM_TB 8
+#define SSM_TB 16
+#define SSM_WHOLE 0
+#define SSM_LOCAL 1
+#define SSM_FROM 2
 
-template <typename T, int NPL>
+// Long portions are cut into chunks of `chunk` tokens that run side by side (the recurrence is linear in the state):
+//   SSM_LOCAL: every chunk from a state of zero, no outputs; leaves its state in ws[chunk] and the sum of its step
+//              sizes in ws_dt[chunk] (the chunk's decay of element n is exp(A[c][n] * that sum))
+//   (ssm_combine_kernel walks a sequence's chunks: ws[j] <- the state in front of chunk j, and the slot's final state)
+//   SSM_FROM:  every chunk again from ws[chunk], writing the outputs
+// SSM_WHOLE is the plain walk from the slot's state.  blockIdx.x = sequence * max_chunks + chunk.
+template <typename T, int NPL, int MODE>
 __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict__ xc, const float* __restrict__ dtp,
                                                              const float* __restrict__ dt_bias, const T* __restrict__ bc,
                                                              int ldbc, int b_col, int c_col, const float* __restrict__ A_log,
@@ -94,15 +105,22 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
                                                              const int* __restrict__ cu_seqlens,
                                                              const int* __restrict__ state_slots, float* __restrict__ state,
                                                              int num_slots, int C, int N, int hist, int LPC,
-                                                             T* __restrict__ out) {
-  const int b = blockIdx.x;
+                                                             T* __restrict__ out, int chunk, int max_chunks,
+                                                             float* __restrict__ ws, float* __restrict__ ws_dt) {
+  extern __shared__ float bcs[];                         // [SSM_TB][2 N]: the block's B and C rows, shared by all channels
+  const int b = MODE == SSM_WHOLE ? blockIdx.x : blockIdx.x / max_chunks;
   const int per = blockDim.x / LPC;                      // channels a workgroup
   const int c = blockIdx.y * per + threadIdx.x / LPC, l = threadIdx.x % LPC;
-  const int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1], slot = state_slots[b];
-  if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;
+  int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
+  const int slot = state_slots[b];
+  if (MODE != SSM_WHOLE) {
+    t_begin += (blockIdx.x % max_chunks) * chunk;
+    t_end = min(t_end, t_begin + chunk);
+  }
+  if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;      // the whole workgroup alike
   const bool c_ok = c < C;
   const int ci = min(c, C - 1);
-  float* sp = state + ((size_t)slot * C + ci) * (N + hist);
+  float* sp = MODE == SSM_WHOLE ? state + ((size_t)slot * C + ci) * (N + hist) : ws + ((size_t)blockIdx.x * C + ci) * N;
   float S[NPL], A[NPL];
   int ni[NPL];
   bool n_ok[NPL];
@@ -111,74 +129,132 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
     const int n = l + j * LPC;
     n_ok[j] = n < N;
     ni[j] = min(n, N - 1);
-    S[j] = n_ok[j] ? sp[ni[j]] : 0.f;
+    S[j] = (MODE != SSM_LOCAL && n_ok[j]) ? sp[ni[j]] : 0.f;
     A[j] = -expf(A_log[(size_t)ci * N + ni[j]]);
   }
   const float bias = dt_bias[ci], Dc = D[ci];
+  float dt_sum = 0.f;
   for (int t0 = t_begin; t0 < t_end; t0 += SSM_TB) {
     const int nb = min(SSM_TB, t_end - t0);
-    float xv[SSM_TB], dv[SSM_TB], zv[SSM_TB], Bv[SSM_TB][NPL], Cv[SSM_TB][NPL];
+    // a thread's own values of the block's tokens travel while the B and C rows are staged
+    float xv[SSM_TB], dv[SSM_TB], zv[SSM_TB];
 #pragma unroll
     for (int k = 0; k < SSM_TB; k++) {
       const size_t t = (size_t)(t0 + min(k, nb - 1));
       xv[k] = load_f32(xc + t * C + ci);
       dv[k] = dtp[t * C + ci];
-      zv[k] = load_f32(z + t * ldz + ci);
-#pragma unroll
-      for (int j = 0; j < NPL; j++) {
-        Bv[k][j] = load_f32(bc + t * ldbc + b_col + ni[j]);
-        Cv[k][j] = load_f32(bc + t * ldbc + c_col + ni[j]);
-      }
+      zv[k] = MODE != SSM_LOCAL ? load_f32(z + t * ldz + ci) : 0.f;
     }
+    __syncthreads();                                     // the last block's rows have been read
+    for (int i = threadIdx.x; i < nb * 2 * N; i += blockDim.x) {
+      const int k = i / (2 * N), e = i % (2 * N);
+      bcs[i] = load_f32(bc + (size_t)(t0 + k) * ldbc + (e < N ? b_col + e : c_col + e - N));
+    }
+    __syncthreads();
 #pragma unroll
     for (int k = 0; k < SSM_TB; k++) {
       if (k >= nb) break;
       const float pre = dv[k] + bias;
       const float dt = pre > 20.f ? pre : log1pf(expf(pre));
       const float dx = dt * xv[k];
+      dt_sum += dt;
+      const float* Bk = bcs + k * 2 * N;
       float y = 0.f;
 #pragma unroll
       for (int j = 0; j < NPL; j++) {
-        S[j] = n_ok[j] ? fmaf(expf(dt * A[j]), S[j], dx * Bv[k][j]) : 0.f;
-        y = fmaf(S[j], Cv[k][j], y);
+        S[j] = n_ok[j] ? fmaf(expf(dt * A[j]), S[j], dx * Bk[ni[j]]) : 0.f;
+        if (MODE != SSM_LOCAL) y = fmaf(S[j], Bk[N + ni[j]], y);
       }
-      for (int off = LPC >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, 64);
-      if (l == 0 && c_ok) store_f32(out + (size_t)(t0 + k) * C + c, fmaf(Dc, xv[k], y) * silu_f(zv[k]));
+      if (MODE != SSM_LOCAL) {
+        for (int off = LPC >> 1; off > 0; off >>= 1) y += __shfl_xor(y, off, 64);
+        if (l == 0 && c_ok) store_f32(out + (size_t)(t0 + k) * C + c, fmaf(Dc, xv[k], y) * silu_f(zv[k]));
+      }
     }
   }
-  if (c_ok) {
+  if (c_ok && MODE != SSM_FROM) {
 #pragma unroll
     for (int j = 0; j < NPL; j++)
       if (n_ok[j]) sp[ni[j]] = S[j];
+    if (MODE == SSM_LOCAL && l == 0) ws_dt[(size_t)blockIdx.x * C + c] = dt_sum;
   }
 }
 
+// The walk over a sequence's chunks, one thread per state element: ws[j] becomes the state in front of chunk j, the
+// slot gets the state behind the last chunk.  grid (sequences, ceil(C N / 256)).
+__global__ __launch_bounds__(256) void ssm_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                                                          float* __restrict__ state, float* __restrict__ ws,
+                                                          const float* __restrict__ ws_dt, const float* __restrict__ A_log,
+                                                          int num_slots, int C, int N, int hist, int chunk, int max_chunks) {
+  const int b = blockIdx.x, e = blockIdx.y * 256 + threadIdx.x;
+  if (e >= C * N) return;
+  const int slot = state_slots[b], n_tok = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || slot >= num_slots || n_tok <= 0) return;
+  const int c = e / N, n = e % N;
+  const float A = -expf(A_log[e]);
+  float* sp = state + ((size_t)slot * C + c) * (N + hist) + n;
+  float S = *sp;
+  const int chunks = (n_tok + chunk - 1) / chunk;
+  for (int j = 0; j < chunks; j++) {
+    const size_t at = (size_t)b * max_chunks + j;
+    float* w = ws + (at * C + c) * N + n;
+    const float local = *w;
+    *w = S;
+    S = fmaf(expf(A * ws_dt[at * C + c]), S, local);
+  }
+  *sp = S;
+}
+
+// chunk == 0: every sequence walked whole from its slot.  chunk > 0: sequences cut into chunks of that many tokens that
+// run side by side (three launches); ws float32 [num_seqs * max_chunks, C, N], ws_dt [num_seqs * max_chunks, C],
+// max_chunks at least the chunks of the longest sequence.
 extern "C" int pico_selective_scan(const void* xc, const float* dtp, const float* dt_bias, const void* bc, int ldbc, int b_col,
                                    int c_col, const float* A_log, const float* D, const void* z, int ldz, int dtype,
                                    const int* cu_seqlens, const int* state_slots, float* state, int num_slots, int B, int T,
-                                   int C, int N, int hist, void* out, hipStream_t stream) {
+                                   int C, int N, int hist, void* out, int chunk, int max_chunks, float* ws, float* ws_dt,
+                                   hipStream_t stream) {
   PICO_REQUIRE(B >= 0 && T >= 0 && C > 0 && N > 0 && N <= 256 && hist >= 0 && num_slots > 0 && ldz >= C &&
                    b_col >= 0 && c_col >= 0 && ldbc >= b_col + N && ldbc >= c_col + N,
                "pico_selective_scan: bad sizes (at most 256 state elements a channel)");
+  PICO_REQUIRE(chunk == 0 || (chunk > 0 && max_chunks > 0 && ws != nullptr && ws_dt != nullptr &&
+                              (long long)max_chunks * chunk >= T && (long long)B * max_chunks < (1ll << 31)),
+               "pico_selective_scan: chunks need room for their states and must cover the step's tokens");
   if (B == 0 || T == 0) return 0;
   int lpc = 1;
-  while (lpc < N && lpc < 64) lpc *= 2;
-  const int npl = (N + lpc - 1) / lpc;                   // 1, 2 or 4 (3 runs as 4)
+  while (lpc * 16 < N) lpc *= 2;                         // up to 16 state elements a lane
+  const int need = (N + lpc - 1) / lpc;
+  const int npl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 8 ? 8 : 16;
+  const size_t lds = (size_t)SSM_TB * 2 * N * sizeof(float);
   const int per = 256 / lpc;
-  const dim3 grid(B, (C + per - 1) / per);
-  PICO_REQUIRE(grid.y <= 65535, "pico_selective_scan: too many channels");
+  const int gy = (C + per - 1) / per;
+  PICO_REQUIRE(gy <= 65535 && ((long long)C * N + 255) / 256 <= 65535, "pico_selective_scan: too many channels");
 #define SSM_ARGS(TT)                                                                                                    \
   (const TT*)xc, dtp, dt_bias, (const TT*)bc, ldbc, b_col, c_col, A_log, D, (const TT*)z, ldz, cu_seqlens, state_slots, \
-      state, num_slots, C, N, hist, lpc, (TT*)out
-#define SSM_LAUNCH(TT)                                                                                    \
-  do {                                                                                                    \
-    if (npl == 1) selective_scan_kernel<TT, 1><<<grid, 256, 0, stream>>>(SSM_ARGS(TT));                   \
-    else if (npl == 2) selective_scan_kernel<TT, 2><<<grid, 256, 0, stream>>>(SSM_ARGS(TT));              \
-    else selective_scan_kernel<TT, 4><<<grid, 256, 0, stream>>>(SSM_ARGS(TT));                            \
+      state, num_slots, C, N, hist, lpc, (TT*)out, chunk, max_chunks, ws, ws_dt
+#define SSM_LAUNCH(TT, MODE, GX)                                                                              \
+  do {                                                                                                        \
+    if (npl == 1) selective_scan_kernel<TT, 1, MODE><<<dim3(GX, gy), 256, lds, stream>>>(SSM_ARGS(TT));       \
+    else if (npl == 2) selective_scan_kernel<TT, 2, MODE><<<dim3(GX, gy), 256, lds, stream>>>(SSM_ARGS(TT));  \
+    else if (npl == 4) selective_scan_kernel<TT, 4, MODE><<<dim3(GX, gy), 256, lds, stream>>>(SSM_ARGS(TT));  \
+    else if (npl == 8) selective_scan_kernel<TT, 8, MODE><<<dim3(GX, gy), 256, lds, stream>>>(SSM_ARGS(TT));  \
+    else selective_scan_kernel<TT, 16, MODE><<<dim3(GX, gy), 256, lds, stream>>>(SSM_ARGS(TT));               \
   } while (0)
-  if (dtype == PICO_DTYPE_F32) SSM_LAUNCH(float);
-  else if (dtype == PICO_DTYPE_BF16) SSM_LAUNCH(bf16_t);
-  else PICO_REQUIRE(false, "pico_selective_scan: unknown dtype %d", dtype);
+#define SSM_RUN(TT)                                                                                                        \
+  if (chunk == 0) {                                                                                                        \
+    SSM_LAUNCH(TT, SSM_WHOLE, B);                                                                                          \
+  } else {                                                                                                                 \
+    SSM_LAUNCH(TT, SSM_LOCAL, B * max_chunks);                                                                             \
+    ssm_combine_kernel<<<dim3(B, (C * N + 255) / 256), 256, 0, stream>>>(cu_seqlens, state_slots, state, ws, ws_dt, A_log, \
+                                                                         num_slots, C, N, hist, chunk, max_chunks);        \
+    SSM_LAUNCH(TT, SSM_FROM, B * max_chunks);                                                                              \
+  }
+  if (dtype == PICO_DTYPE_F32) {
+    SSM_RUN(float)
+  } else if (dtype == PICO_DTYPE_BF16) {
+    SSM_RUN(bf16_t)
+  } else {
+    PICO_REQUIRE(false, "pico_selective_scan: unknown dtype %d", dtype);
+  }
+#undef SSM_RUN
 #undef SSM_LAUNCH
 #undef SSM_ARGS
   PICO_LAUNCH_CHECK();

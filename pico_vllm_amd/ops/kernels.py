@@ -1128,11 +1128,14 @@ def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Ten
 
 
 def selective_scan(xc: torch.Tensor, dt_pre: torch.Tensor, dt_bias: torch.Tensor, bc: torch.Tensor, b_col: int, c_col: int,
-                   a_log: torch.Tensor, d: torch.Tensor, z: torch.Tensor, ctx, state: torch.Tensor, hist: int) -> torch.Tensor:
+                   a_log: torch.Tensor, d: torch.Tensor, z: torch.Tensor, ctx, state: torch.Tensor, hist: int,
+                   chunk: int = 0) -> torch.Tensor:
     """The recurrence S <- exp(dt A) S + dt x B, y = S . C + D x with dt = softplus(dt_pre + dt_bias), A = -exp(a_log), for
     every sequence of the step from its state slot (``state`` float32 [slots, channels, N + hist], updated in place);
     returns y * silu(z) [T, channels] in xc's dtype.  xc [T, channels]; dt_pre float32 [T, channels]; B and C are
-    columns b_col .. and c_col .. of ``bc``; z [T, >= channels] (row stride free)."""
+    columns b_col .. and c_col .. of ``bc``; z [T, >= channels] (row stride free).
+    ``chunk`` > 0: sequences are cut into chunks of that many tokens that run side by side (every chunk from zero, a walk
+    over the chunks' states, every chunk again from its true state): the same sums in another order."""
     _gpu(xc, dt_pre, dt_bias, bc, a_log, d, z, state)
     T, C = xc.shape
     N = a_log.shape[1]
@@ -1150,11 +1153,17 @@ def selective_scan(xc: torch.Tensor, dt_pre: torch.Tensor, dt_bias: torch.Tensor
     B = ctx.num_seqs
     _i32(ctx.cu_seqlens, "cu_seqlens", B + 1); _i32(ctx.state_slots, "state_slots", B)
     out = torch.empty(T, C, dtype=xc.dtype, device=xc.device)
+    ws = ws_dt = None
+    max_chunks = 0
+    if chunk > 0:
+        max_chunks = -(-T // chunk)
+        ws = torch.empty(B * max_chunks, C, N, dtype=torch.float32, device=xc.device)
+        ws_dt = torch.empty(B * max_chunks, C, dtype=torch.float32, device=xc.device)
     lib = library.core()
     _check(lib, lib.pico_selective_scan(_ptr(xc), _ptr(dt_pre), _ptr(dt_bias), _ptr(bc), bc.stride(0) if T > 1 else bc.shape[1],
                                         b_col, c_col, _ptr(a_log), _ptr(d), _ptr(z), z.stride(0) if T > 1 else z.shape[1], _dt(xc),
                                         _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(state), state.shape[0], B, T, C, N, hist,
-                                        _ptr(out), _stream()))
+                                        _ptr(out), chunk, max_chunks, _ptr(ws), _ptr(ws_dt), _stream()))
     return out
 
 

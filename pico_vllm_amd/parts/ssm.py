@@ -27,6 +27,11 @@ class SelectiveStateSpace(Mixer):
 
     graph_safe_prompts = True
 
+    # In the bfloat16 engine a step with a prompt portion cuts its sequences into chunks of this many tokens that run
+    # side by side (``kernels.selective_scan``); decided from the step's shape alone.  The 32-bit engine walks every
+    # sequence whole, so that its sums do not depend on how a prompt was cut.
+    CHUNK, CHUNKED_FROM = 64, 128
+
     NAMES = {"in": "in", "conv": "conv", "conv_bias": "conv.b", "x": "x", "dt": "dt", "dt_bias": "dt.b", "a_log": "A_log",
              "d": "D", "o": "o"}
 
@@ -75,5 +80,6 @@ class SelectiveStateSpace(Mixer):
         u = kernels.causal_conv(uz, I, self.conv_w, self.conv_b, ctx, cache.state, N)
         dbc = self.x_proj(u)                                                         # [T, d | B | C]
         dt_pre = self.dt_proj(dbc[:, :R], out_dtype=torch.float32)                   # step sizes stay float32 from here on
+        chunked = self.act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= self.CHUNKED_FROM
         return kernels.selective_scan(u, dt_pre, self.dt_bias, dbc, R, R + N, self.a_log, self.d, uz[:, I:], ctx, cache.state,
-                                      self.taps - 1)
+                                      self.taps - 1, chunk=self.CHUNK if chunked else 0)

@@ -228,7 +228,7 @@ def test_a_product_per_head(dtype, T, H, n_in, n_out, copy):
 @pytest.mark.parametrize("C,N,taps,R", [(100, 12, 3, 5), (256, 16, 4, 8), (160, 80, 2, 7), (36, 5, 1, 3), (40, 200, 5, 4)])
 def test_convolution_and_recurrence_in_portions_and_token_by_token(dtype, C, N, taps, R):
     """Three sequences in slots that were used before (zeroed as the engine does for a new request): whole, in portions
-    down to one token beside each other, against the plain walk."""
+    down to one token beside each other, and cut into chunks that run side by side, against the plain walk."""
     from pico_vllm_amd.ops import kernels
     g = torch.Generator().manual_seed(C + N)
     lens = [37, 5, 18]
@@ -246,7 +246,10 @@ def test_convolution_and_recurrence_in_portions_and_token_by_token(dtype, C, N, 
         y, _ = P.selective_scan(u, dt, -torch.exp(a_log.double()), s["dbc"][:, R:R + N].double(), s["dbc"][:, R + N:].double(), D.double())
         want.append((u, y * P.silu(s["uz"][:, C:].double())))
     dev = lambda t: t.to(DEV).contiguous()
-    for portions in ([[37, 5, 18]], [[2, 1, 7], [30, 3, 1], [1, 1, 9], [4, 0, 1]], [[1, 1, 1]] * 5 + [[32, 0, 13]]):
+    plans = [([[37, 5, 18]], 0), ([[2, 1, 7], [30, 3, 1], [1, 1, 9], [4, 0, 1]], 0), ([[1, 1, 1]] * 5 + [[32, 0, 13]], 0)]
+    if dtype == "bfloat16":          # chunks that run side by side: of 4 and of 16 tokens, sequences of unequal numbers of chunks
+        plans += [([[37, 5, 18]], 4), ([[20, 2, 1], [17, 3, 17]], 16)]
+    for portions, chunk in plans:
         state = torch.full((5, C, N + taps - 1), 9.0, device=DEV)
         slots = [4, 0, 2]
         state[slots] = 0
@@ -257,7 +260,7 @@ def test_convolution_and_recurrence_in_portions_and_token_by_token(dtype, C, N, 
             cat = lambda k: dev(torch.cat([seqs[b][k][fed[b]:fed[b] + step[b]] for b in live]))
             uz, dbc, dtp = cat("uz"), cat("dbc"), cat("dtp")
             u = kernels.causal_conv(uz, C, dev(w), dev(cb), ctx, state, N)
-            y = kernels.selective_scan(u, dtp, dev(dtb), dbc, R, R + N, dev(a_log), dev(D), uz[:, C:], ctx, state, taps - 1)
+            y = kernels.selective_scan(u, dtp, dev(dtb), dbc, R, R + N, dev(a_log), dev(D), uz[:, C:], ctx, state, taps - 1, chunk=chunk)
             at = 0
             for b in live:
                 got_u[b].append(u[at:at + step[b]])
