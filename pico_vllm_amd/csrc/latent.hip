@@ -106,38 +106,47 @@ extern "C" int pico_rope_inplace(void* x, int ldx, int dtype, int col0, int head
 // ---------------------------------------------------------------------------
 // A product per head: out[t][h][o] = sum_i x[t][h][i] * W[h][i][o]        (W [heads, in, out]: a head's matrix with the
 // inner index first, so that neighbouring threads read neighbouring addresses)
-// x: head h of row t at x + t ldx + x_col + h x_head;  out likewise.  grid (T, heads, tiles of 128 outputs); the sum's order
+// x: head h of row t at x + t ldx + x_col + h x_head;  out likewise.  grid (T, heads, tiles of 64 outputs); the sum's order
 // depends on `in` alone.
 // `copy` > 0: the `copy` entries behind a head's `in` inputs are handed on behind its `out` outputs (a rotated part
 // that goes on as it is).
 // ---------------------------------------------------------------------------
-#define HEAD_LINEAR_TILE 128
+#define HEAD_LINEAR_TILE 64
+#define HEAD_LINEAR_SLICES 4
+// A workgroup makes HEAD_LINEAR_TILE outputs of one head of one token; its four waves take a quarter of the inner
+// index each (so that a matrix's loads travel side by side, not one behind the other) and their partial sums meet in
+// LDS and are added in the waves' order: the sum's order depends on `in` alone.
 template <typename T>
-__global__ __launch_bounds__(HEAD_LINEAR_TILE) void head_linear_kernel(const T* __restrict__ x, int ldx, int x_col, int x_head,
-                                                                       const T* __restrict__ W, T* __restrict__ out, int ldo,
-                                                                       int o_col, int o_head, int in, int outn, int copy) {
-  extern __shared__ float xs[];
+__global__ __launch_bounds__(HEAD_LINEAR_TILE* HEAD_LINEAR_SLICES) void head_linear_kernel(
+    const T* __restrict__ x, int ldx, int x_col, int x_head, const T* __restrict__ W, T* __restrict__ out, int ldo, int o_col,
+    int o_head, int in, int outn, int copy) {
+  extern __shared__ float xs[];                           // [in + copy], then [slices][tile] partial sums
   const int t = blockIdx.x, h = blockIdx.y;
   const T* xr = x + (size_t)t * ldx + x_col + (size_t)h * x_head;
   const int extra = blockIdx.z == 0 ? copy : 0;          // the first tile of a head hands the copied entries on
   for (int i = threadIdx.x; i < in + extra; i += blockDim.x) xs[i] = load_f32(xr + i);
   __syncthreads();
+  float* part = xs + in + copy;
   const T* w = W + (size_t)h * in * outn;
   T* o = out + (size_t)t * ldo + o_col + (size_t)h * o_head;
-  const int c = blockIdx.z * HEAD_LINEAR_TILE + threadIdx.x;
-  if (c < outn) {
-    // four chains over i mod 4, added at the end: the order depends on `in` alone
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int i = 0;
-    for (; i + 3 < in; i += 4) {
-      a0 = fmaf(xs[i], load_f32(w + (size_t)i * outn + c), a0);
-      a1 = fmaf(xs[i + 1], load_f32(w + (size_t)(i + 1) * outn + c), a1);
-      a2 = fmaf(xs[i + 2], load_f32(w + (size_t)(i + 2) * outn + c), a2);
-      a3 = fmaf(xs[i + 3], load_f32(w + (size_t)(i + 3) * outn + c), a3);
-    }
-    for (; i < in; i++) a0 = fmaf(xs[i], load_f32(w + (size_t)i * outn + c), a0);
-    store_f32(o + c, (a0 + a1) + (a2 + a3));
+  const int cx = threadIdx.x % HEAD_LINEAR_TILE, slice = threadIdx.x / HEAD_LINEAR_TILE;
+  const int c = blockIdx.z * HEAD_LINEAR_TILE + cx, cc = min(c, outn - 1);
+  const int per = (in + HEAD_LINEAR_SLICES - 1) / HEAD_LINEAR_SLICES;
+  const int i0 = slice * per, i1 = min(in, i0 + per);
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  int i = i0;
+#pragma unroll 2
+  for (; i + 3 < i1; i += 4) {
+    a0 = fmaf(xs[i], load_f32(w + (size_t)i * outn + cc), a0);
+    a1 = fmaf(xs[i + 1], load_f32(w + (size_t)(i + 1) * outn + cc), a1);
+    a2 = fmaf(xs[i + 2], load_f32(w + (size_t)(i + 2) * outn + cc), a2);
+    a3 = fmaf(xs[i + 3], load_f32(w + (size_t)(i + 3) * outn + cc), a3);
   }
+  for (; i < i1; i++) a0 = fmaf(xs[i], load_f32(w + (size_t)i * outn + cc), a0);
+  part[slice * HEAD_LINEAR_TILE + cx] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (slice == 0 && c < outn)
+    store_f32(o + c, (part[cx] + part[HEAD_LINEAR_TILE + cx]) + (part[2 * HEAD_LINEAR_TILE + cx] + part[3 * HEAD_LINEAR_TILE + cx]));
   for (int k = threadIdx.x; k < extra; k += blockDim.x) store_f32(o + outn + k, xs[in + k]);
 }
 
@@ -148,13 +157,13 @@ extern "C" int pico_head_linear(const void* x, int ldx, int x_col, int x_head, c
   PICO_REQUIRE(ldx >= x_col + (heads - 1) * x_head + in + copy && ldo >= o_col + (heads - 1) * o_head + outn + copy,
                "pico_head_linear: the heads do not fit the rows");
   if (T == 0) return 0;
-  const size_t lds = (size_t)(in + copy) * sizeof(float);
+  const size_t lds = (size_t)(in + copy + HEAD_LINEAR_TILE * HEAD_LINEAR_SLICES) * sizeof(float);
   const int tiles = (outn + HEAD_LINEAR_TILE - 1) / HEAD_LINEAR_TILE;
   if (dtype == PICO_DTYPE_F32)
-    head_linear_kernel<float><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE, lds, stream>>>((const float*)x, ldx, x_col, x_head, (const float*)W,
+    head_linear_kernel<float><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE * HEAD_LINEAR_SLICES, lds, stream>>>((const float*)x, ldx, x_col, x_head, (const float*)W,
                                                                     (float*)out, ldo, o_col, o_head, in, outn, copy);
   else if (dtype == PICO_DTYPE_BF16)
-    head_linear_kernel<bf16_t><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE, lds, stream>>>((const bf16_t*)x, ldx, x_col, x_head, (const bf16_t*)W,
+    head_linear_kernel<bf16_t><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE * HEAD_LINEAR_SLICES, lds, stream>>>((const bf16_t*)x, ldx, x_col, x_head, (const bf16_t*)W,
                                                                      (bf16_t*)out, ldo, o_col, o_head, in, outn, copy);
   else
     PICO_REQUIRE(false, "pico_head_linear: unknown dtype %d", dtype);

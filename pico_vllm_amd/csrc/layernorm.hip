@@ -9,38 +9,91 @@
 
 #define LN_MAX_SLABS 16
 
-template <typename TD, typename TO>
-__global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta, int slabs,
-                                                            size_t slab_stride, const float* __restrict__ dscale,
-                                                            const float* __restrict__ w, const float* __restrict__ b,
-                                                            TO* __restrict__ out, const int* __restrict__ rows, int H,
-                                                            float eps) {
+// One workgroup a row.  VEC: four elements a thread and turn with 16-byte accesses (H a multiple of 4, everything
+// aligned); the row is kept in LDS between the passes.
+template <typename TD> __device__ __forceinline__ float4 ln_load4(const TD* p);
+template <> __device__ __forceinline__ float4 ln_load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 ln_load4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+template <typename TO> __device__ __forceinline__ void ln_store4(TO* p, float4 v);
+template <> __device__ __forceinline__ void ln_store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void ln_store4<bf16_t>(bf16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w));
+}
+
+template <typename TD, typename TO, bool VEC>
+__global__ __launch_bounds__(1024) void add_layernorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta, int slabs,
+                                                             size_t slab_stride, const float* __restrict__ dscale,
+                                                             const float* __restrict__ w, const float* __restrict__ b,
+                                                             TO* __restrict__ out, const int* __restrict__ rows, int H,
+                                                             float eps) {
   extern __shared__ float xs[];          // [H] the row, then 16 floats of scratch
   float* scratch = xs + H;
   const int row = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)row * H;
   const TD* dl = delta ? delta + (size_t)row * H : nullptr;
+  TO* o = out + (size_t)blockIdx.x * H;
   float s = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = x[i];
-    if (dl) {
-      float d = load_f32(dl + i);
-      for (int k = 1; k < slabs; k++) d += load_f32(dl + k * slab_stride + i);
-      v += dscale ? dscale[i] * d : d;
-      if (!rows) x[i] = v;
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(x + i);
+      if (dl) {
+        float4 d = ln_load4<TD>(dl + i);
+        for (int k = 1; k < slabs; k++) {
+          const float4 e = ln_load4<TD>(dl + k * slab_stride + i);
+          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+        }
+        if (dscale) {
+          const float4 c = *reinterpret_cast<const float4*>(dscale + i);
+          d.x *= c.x; d.y *= c.y; d.z *= c.z; d.w *= c.w;
+        }
+        v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        if (!rows) *reinterpret_cast<float4*>(x + i) = v;
+      }
+      *reinterpret_cast<float4*>(xs + i) = v;
+      s += (v.x + v.y) + (v.z + v.w);
     }
-    xs[i] = v;
-    s += v;
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float v = x[i];
+      if (dl) {
+        float d = load_f32(dl + i);
+        for (int k = 1; k < slabs; k++) d += load_f32(dl + k * slab_stride + i);
+        v += dscale ? dscale[i] * d : d;
+        if (!rows) x[i] = v;
+      }
+      xs[i] = v;
+      s += v;
+    }
   }
   const float mean = block_sum(s, scratch) / (float)H;
   float q = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float d = xs[i] - mean;
-    q = fmaf(d, d, q);
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(xs + i);
+      const float d0 = v.x - mean, d1 = v.y - mean, d2 = v.z - mean, d3 = v.w - mean;
+      q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      const float d = xs[i] - mean;
+      q = fmaf(d, d, q);
+    }
   }
   const float r = 1.0f / sqrtf(block_sum(q, scratch) / (float)H + eps);
-  TO* o = out + (size_t)blockIdx.x * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(o + i, (xs[i] - mean) * r * w[i] + b[i]);
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(xs + i);
+      const float4 g = *reinterpret_cast<const float4*>(w + i), c = *reinterpret_cast<const float4*>(b + i);
+      ln_store4<TO>(o + i, make_float4((v.x - mean) * r * g.x + c.x, (v.y - mean) * r * g.y + c.y, (v.z - mean) * r * g.z + c.z,
+                                       (v.w - mean) * r * g.w + c.w));
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(o + i, (xs[i] - mean) * r * w[i] + b[i]);
+  }
 }
 
 extern "C" int pico_add_layernorm(float* resid, const void* delta, int delta_dtype, int slabs, long long slab_stride,
@@ -51,9 +104,18 @@ extern "C" int pico_add_layernorm(float* resid, const void* delta, int delta_dty
   PICO_REQUIRE(eps > 0.f && w != nullptr && b != nullptr, "pico_add_layernorm: eps must be positive, weight and bias given");
   if (T == 0) return 0;
   const size_t lds = (size_t)(H + 16) * sizeof(float);
-#define LAUNCH(TD, TO)                                                                                                   \
-  add_layernorm_kernel<TD, TO><<<T, 256, lds, stream>>>(resid, (const TD*)delta, slabs, (size_t)slab_stride, dscale, w, \
-                                                        b, (TO*)out, rows, H, eps)
+  const bool vec = H % 4 == 0 && slab_stride % 4 == 0 && (uintptr_t)resid % 16 == 0 && (uintptr_t)delta % 16 == 0 &&
+                   (uintptr_t)dscale % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)b % 16 == 0 && (uintptr_t)out % 16 == 0;
+  const int threads = vec ? min(1024, max(64, (H / 4 + 63) / 64 * 64)) : min(1024, max(64, (H + 63) / 64 * 64));
+#define LAUNCH(TD, TO)                                                                                                    \
+  do {                                                                                                                    \
+    if (vec)                                                                                                              \
+      add_layernorm_kernel<TD, TO, true><<<T, threads, lds, stream>>>(resid, (const TD*)delta, slabs, (size_t)slab_stride, \
+                                                                      dscale, w, b, (TO*)out, rows, H, eps);              \
+    else                                                                                                                  \
+      add_layernorm_kernel<TD, TO, false><<<T, threads, lds, stream>>>(resid, (const TD*)delta, slabs, (size_t)slab_stride, \
+                                                                       dscale, w, b, (TO*)out, rows, H, eps);             \
+  } while (0)
   if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_F32) LAUNCH(float, float);
   else if (delta_dtype == PICO_DTYPE_BF16 && out_dtype == PICO_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == PICO_DTYPE_F32 && out_dtype == PICO_DTYPE_BF16) LAUNCH(float, bf16_t);

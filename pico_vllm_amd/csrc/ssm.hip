@@ -14,6 +14,11 @@
 #define SSM_MAX_TAPS 16
 
 __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+// the decay exp(dt A) of an element: the library's exponential in the 32-bit engine; with bfloat16 storage the
+// hardware's (exp2 of the argument times log2 e; the argument is at most 0, the relative error a few 1e-7)
+template <typename T> __device__ __forceinline__ float decay_exp(float v);
+template <> __device__ __forceinline__ float decay_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float decay_exp<bf16_t>(float v) { return __expf(v); }
 
 // grid (T, ceil(C / 256)): one thread per (token, channel).  Inputs before the portion come from the slot's history.
 template <typename T>
@@ -162,7 +167,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
       float y = 0.f;
 #pragma unroll
       for (int j = 0; j < NPL; j++) {
-        S[j] = n_ok[j] ? fmaf(expf(dt * A[j]), S[j], dx * Bk[ni[j]]) : 0.f;
+        S[j] = n_ok[j] ? fmaf(decay_exp<T>(dt * A[j]), S[j], dx * Bk[ni[j]]) : 0.f;
         if (MODE != SSM_LOCAL) y = fmaf(S[j], Bk[N + ni[j]], y);
       }
       if (MODE != SSM_LOCAL) {

@@ -23,7 +23,7 @@ BOUND = {"float32": 3e-5, "bfloat16": 7e-2}
 # (The margin is counted in units of the router logits' spread over a row; what reaches a router after several layer
 # runs in bfloat16 is off by a few percent of its size, and so are the logits.)
 CLOSE_CALL, TAINTED_BOUND = 0.25, 2.5
-FLOAT32_CLOSE, FLOAT32_LOOSE = 0.002, 1e-3
+FLOAT32_CLOSE, FLOAT32_LOOSE = 0.01, 1e-3
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 PAGE = {"a": 16, "b": 8, "c": 32, "d": 16}
 
