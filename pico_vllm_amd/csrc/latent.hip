@@ -109,7 +109,7 @@ extern "C" int pico_rope_inplace(void* x, int ldx, int dtype, int col0, int head
 // x: head h of row t at x + t ldx + x_col + h x_head;  out likewise.  grid (T, heads, tiles of 64 outputs); the sum's order
 // depends on `in` alone.
 // `copy` > 0: the `copy` entries behind a head's `in` inputs are handed on behind its `out` outputs (a rotated part
-// that goes on as it is).
+// that goes on as it is, or is turned on the way).
 // ---------------------------------------------------------------------------
 #define HEAD_LINEAR_TILE 64
 #define HEAD_LINEAR_SLICES 4
@@ -119,7 +119,7 @@ extern "C" int pico_rope_inplace(void* x, int ldx, int dtype, int col0, int head
 template <typename T>
 __global__ __launch_bounds__(HEAD_LINEAR_TILE* HEAD_LINEAR_SLICES) void head_linear_kernel(
     const T* __restrict__ x, int ldx, int x_col, int x_head, const T* __restrict__ W, T* __restrict__ out, int ldo, int o_col,
-    int o_head, int in, int outn, int copy) {
+    int o_head, int in, int outn, int copy, const float* __restrict__ cos_sin) {
   extern __shared__ float xs[];                           // [in + copy], then [slices][tile] partial sums
   const int t = blockIdx.x, h = blockIdx.y;
   const T* xr = x + (size_t)t * ldx + x_col + (size_t)h * x_head;
@@ -147,11 +147,23 @@ __global__ __launch_bounds__(HEAD_LINEAR_TILE* HEAD_LINEAR_SLICES) void head_lin
   __syncthreads();
   if (slice == 0 && c < outn)
     store_f32(o + c, (part[cx] + part[HEAD_LINEAR_TILE + cx]) + (part[2 * HEAD_LINEAR_TILE + cx] + part[3 * HEAD_LINEAR_TILE + cx]));
-  for (int k = threadIdx.x; k < extra; k += blockDim.x) store_f32(o + outn + k, xs[in + k]);
+  // the copied entries as they are, or (cos_sin given: [T, copy / 2, 2]) turned by the token's angles, neighbours in pairs
+  const float* cs = cos_sin ? cos_sin + (size_t)t * copy : nullptr;
+  for (int k = threadIdx.x; k < extra; k += blockDim.x) {
+    float v = xs[in + k];
+    if (cs) {
+      const int p = k >> 1;
+      const float a = xs[in + 2 * p], b = xs[in + 2 * p + 1], c = cs[2 * p], sn = cs[2 * p + 1];
+      v = (k & 1) ? b * c + a * sn : a * c - b * sn;
+    }
+    store_f32(o + outn + k, v);
+  }
 }
 
 extern "C" int pico_head_linear(const void* x, int ldx, int x_col, int x_head, const void* W, void* out, int ldo, int o_col,
-                                int o_head, int dtype, int T, int heads, int in, int outn, int copy, hipStream_t stream) {
+                                int o_head, int dtype, int T, int heads, int in, int outn, int copy, const float* cos_sin,
+                                hipStream_t stream) {
+  PICO_REQUIRE(cos_sin == nullptr || copy % 2 == 0, "pico_head_linear: a part that is turned has an even number of entries");
   PICO_REQUIRE(T >= 0 && heads > 0 && heads <= 65535 && in > 0 && outn > 0 && copy >= 0 && in + copy <= 12288,
                "pico_head_linear: bad sizes");
   PICO_REQUIRE(ldx >= x_col + (heads - 1) * x_head + in + copy && ldo >= o_col + (heads - 1) * o_head + outn + copy,
@@ -161,10 +173,10 @@ extern "C" int pico_head_linear(const void* x, int ldx, int x_col, int x_head, c
   const int tiles = (outn + HEAD_LINEAR_TILE - 1) / HEAD_LINEAR_TILE;
   if (dtype == PICO_DTYPE_F32)
     head_linear_kernel<float><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE * HEAD_LINEAR_SLICES, lds, stream>>>((const float*)x, ldx, x_col, x_head, (const float*)W,
-                                                                    (float*)out, ldo, o_col, o_head, in, outn, copy);
+                                                                    (float*)out, ldo, o_col, o_head, in, outn, copy, cos_sin);
   else if (dtype == PICO_DTYPE_BF16)
     head_linear_kernel<bf16_t><<<dim3(T, heads, tiles), HEAD_LINEAR_TILE * HEAD_LINEAR_SLICES, lds, stream>>>((const bf16_t*)x, ldx, x_col, x_head, (const bf16_t*)W,
-                                                                     (bf16_t*)out, ldo, o_col, o_head, in, outn, copy);
+                                                                     (bf16_t*)out, ldo, o_col, o_head, in, outn, copy, cos_sin);
   else
     PICO_REQUIRE(false, "pico_head_linear: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

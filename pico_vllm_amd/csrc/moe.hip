@@ -358,35 +358,40 @@ extern "C" int pico_moe_experts_plain(const void* h, int ldh, int dtype, const v
 // whose logits are made in the same launch and take no part in the choice (a gate of the layer, say): z is
 // [T, E + extra], and what the choice reads of it has the bias added.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void moe_route_top_softmax_kernel(float* __restrict__ z, const float* __restrict__ bias,
-                                                                   int T, int E, int ldz, int top,
-                                                                   int* __restrict__ experts, float* __restrict__ weights) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+// A wave a token, four tokens a workgroup; lane l looks after logits l, l + 64, ..: it keeps them (bias added) in LDS,
+// where it alone reads and writes them, so the waves never wait for one another.
+__global__ __launch_bounds__(256) void moe_route_top_softmax_kernel(float* __restrict__ z, const float* __restrict__ bias,
+                                                                    int T, int E, int ldz, int top,
+                                                                    int* __restrict__ experts, float* __restrict__ weights) {
+  extern __shared__ float zs[];                          // [4][E]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   float* row = z + (size_t)t * ldz;
-  if (bias)
-    for (int e = 0; e < E; e++) row[e] += bias[e];
-  int chosen[MOE_MAX_TOP];
-  float val[MOE_MAX_TOP];
-  for (int k = 0; k < top; k++) {
-    int best = -1;
-    float bz = 0.f;
-    for (int e = 0; e < E; e++) {
-      bool taken = false;
-      for (int j = 0; j < k; j++) taken |= chosen[j] == e;
-      if (taken) continue;
-      const float v = row[e];
-      if (best < 0 || v > bz) { best = e; bz = v; }
-    }
-    chosen[k] = best;
-    val[k] = bz;
+  float* mine = zs + (size_t)wave * E;
+  for (int e = lane; e < E; e += 64) {
+    const float v = row[e] + (bias ? bias[e] : 0.f);
+    row[e] = v;
+    mine[e] = v;
   }
-  const float largest = val[0];
-  float sum = 0.f;
-  for (int k = 0; k < top; k++) { val[k] = expf(val[k] - largest); sum += val[k]; }
+  float wk = 0.f, largest = 0.f, sum = 0.f;              // lane k keeps the k-th chosen logit's weight
+  int ek = 0;
   for (int k = 0; k < top; k++) {
-    experts[(size_t)t * top + k] = chosen[k];
-    weights[(size_t)t * top + k] = val[k] / sum;
+    float mx = -INFINITY;
+    int mi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = mine[e];
+      if (v > mx || mi == 0x7fffffff) { mx = v; mi = e; }      // the first of equals stays; NaN never wins over a number
+    }
+    wave_first_max(mx, mi);                              // the lowest index among equal values, in every lane
+    if (k == 0) largest = mx;
+    const float w = expf(mx - largest);
+    sum += w;
+    if (lane == k) { wk = w; ek = mi; }
+    if ((mi & 63) == lane) mine[mi] = -INFINITY;         // taken
+  }
+  if (lane < top) {
+    experts[(size_t)t * top + lane] = ek;
+    weights[(size_t)t * top + lane] = wk / sum;
   }
 }
 
@@ -406,7 +411,8 @@ extern "C" int pico_moe_router_top_softmax(const void* x, int ldx, int dtype, co
   if (dtype == PICO_DTYPE_F32) { if (vec) LAUNCH(float, true); else LAUNCH(float, false); }
   else { if (vec) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
 #undef LAUNCH
-  moe_route_top_softmax_kernel<<<(T + 63) / 64, 64, 0, stream>>>(z, bias, T, E, rows, top, experts, weights);
+  PICO_REQUIRE(E <= 8192, "pico_moe_router_top_softmax: at most 8192 experts");
+  moe_route_top_softmax_kernel<<<(T + 3) / 4, 256, (size_t)4 * E * sizeof(float), stream>>>(z, bias, T, E, rows, top, experts, weights);
   PICO_LAUNCH_CHECK();
   return 0;
 }

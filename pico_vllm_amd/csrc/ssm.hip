@@ -41,6 +41,44 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
   store_f32(out + (size_t)t * C + c, silu_f(acc));
 }
 
+// The same for bfloat16 with eight neighbouring channels a thread (16-byte accesses; C and the row stride multiples of 8).
+// grid (T, ceil(C / 8 / 256)).
+__global__ __launch_bounds__(256) void causal_conv8_kernel(const bf16_t* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                           const float* __restrict__ bias, const int* __restrict__ token_seq,
+                                                           const int* __restrict__ cu_seqlens,
+                                                           const int* __restrict__ state_slots, const float* __restrict__ state,
+                                                           int num_slots, int C, int N, int taps, bf16_t* __restrict__ out) {
+  const int t = blockIdx.x, c0 = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c0 >= C) return;
+  const int b = token_seq[t], first = cu_seqlens[b];
+  const int slot = min(max(state_slots[b], 0), num_slots - 1);
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = bias[c0 + i];
+  for (int j = 0; j < taps; j++) {
+    const int src = t - (taps - 1) + j;
+    float v[8];
+    if (src >= first) {
+      const uint4 r = *reinterpret_cast<const uint4*>(x + (size_t)src * ldx + c0);
+      v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+      v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+      v[4] = __uint_as_float(r.z << 16); v[5] = __uint_as_float(r.z & 0xffff0000u);
+      v[6] = __uint_as_float(r.w << 16); v[7] = __uint_as_float(r.w & 0xffff0000u);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = state[((size_t)slot * C + c0 + i) * (N + taps - 1) + N + (taps - 1) + (src - first)];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = fmaf(w[(size_t)(c0 + i) * taps + j], v[i], acc[i]);
+  }
+  uint4 o;
+  o.x = pack2_bf16(silu_f(acc[0]), silu_f(acc[1]));
+  o.y = pack2_bf16(silu_f(acc[2]), silu_f(acc[3]));
+  o.z = pack2_bf16(silu_f(acc[4]), silu_f(acc[5]));
+  o.w = pack2_bf16(silu_f(acc[6]), silu_f(acc[7]));
+  *reinterpret_cast<uint4*>(out + (size_t)t * C + c0) = o;
+}
+
 // grid (sequences, ceil(C / 256)): the slot's history becomes the last taps - 1 inputs behind this step's tokens.
 template <typename T>
 __global__ __launch_bounds__(256) void conv_history_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ cu_seqlens,
@@ -59,22 +97,64 @@ __global__ __launch_bounds__(256) void conv_history_kernel(const T* __restrict__
   for (int k = 0; k < taps - 1; k++) hist[k] = keep[k];
 }
 
+// Every sequence brings ONE token (a decode step): convolution and history in one launch, a thread per (sequence,
+// channel), which reads its history before it writes it.  grid (sequences, ceil(C / 256)).
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_step_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                               const float* __restrict__ bias, const int* __restrict__ cu_seqlens,
+                                                               const int* __restrict__ state_slots, float* __restrict__ state,
+                                                               int num_slots, int C, int N, int taps, T* __restrict__ out) {
+  const int b = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int t = cu_seqlens[b], slot = state_slots[b];
+  if (cu_seqlens[b + 1] != t + 1 || slot < 0 || slot >= num_slots) return;
+  float* hist = state + ((size_t)slot * C + c) * (N + taps - 1) + N;
+  const float xv = load_f32(x + (size_t)t * ldx + c);
+  float acc = bias[c];
+  float keep[SSM_MAX_TAPS];
+  for (int j = 0; j < taps - 1; j++) {
+    keep[j] = hist[j];
+    acc = fmaf(w[(size_t)c * taps + j], keep[j], acc);
+  }
+  acc = fmaf(w[(size_t)c * taps + taps - 1], xv, acc);
+  for (int j = 0; j + 1 < taps - 1; j++) hist[j] = keep[j + 1];
+  if (taps > 1) hist[taps - 2] = xv;
+  store_f32(out + (size_t)t * C + c, silu_f(acc));
+}
+
 extern "C" int pico_causal_conv(const void* x, int ldx, int dtype, const float* w, const float* bias, const int* token_seq,
                                 const int* cu_seqlens, const int* state_slots, float* state, int num_slots, int T, int B,
-                                int C, int N, int taps, void* out, hipStream_t stream) {
+                                int C, int N, int taps, void* out, int single, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && B >= 0 && C > 0 && N > 0 && taps >= 1 && taps <= SSM_MAX_TAPS && ldx >= C && num_slots > 0,
                "pico_causal_conv: bad sizes (1 to %d taps)", SSM_MAX_TAPS);
   if (T == 0 || B == 0) return 0;
   const int cb = (C + 255) / 256;
   PICO_REQUIRE(cb <= 65535, "pico_causal_conv: too many channels");
+  if (single) {               // one token a sequence (the caller says so; a sequence of another length is left alone)
+    PICO_REQUIRE(T == B, "pico_causal_conv: a step of single tokens has as many tokens as sequences");
+    if (dtype == PICO_DTYPE_F32)
+      causal_conv_step_kernel<float><<<dim3(B, cb), 256, 0, stream>>>((const float*)x, ldx, w, bias, cu_seqlens, state_slots, state,
+                                                                      num_slots, C, N, taps, (float*)out);
+    else if (dtype == PICO_DTYPE_BF16)
+      causal_conv_step_kernel<bf16_t><<<dim3(B, cb), 256, 0, stream>>>((const bf16_t*)x, ldx, w, bias, cu_seqlens, state_slots, state,
+                                                                       num_slots, C, N, taps, (bf16_t*)out);
+    else
+      PICO_REQUIRE(false, "pico_causal_conv: unknown dtype %d", dtype);
+    PICO_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == PICO_DTYPE_F32) {
     causal_conv_kernel<float><<<dim3(T, cb), 256, 0, stream>>>((const float*)x, ldx, w, bias, token_seq, cu_seqlens, state_slots,
                                                                state, num_slots, C, N, taps, (float*)out);
     if (taps > 1)
       conv_history_kernel<float><<<dim3(B, cb), 256, 0, stream>>>((const float*)x, ldx, cu_seqlens, state_slots, state, num_slots, C, N, taps);
   } else if (dtype == PICO_DTYPE_BF16) {
-    causal_conv_kernel<bf16_t><<<dim3(T, cb), 256, 0, stream>>>((const bf16_t*)x, ldx, w, bias, token_seq, cu_seqlens, state_slots,
-                                                                state, num_slots, C, N, taps, (bf16_t*)out);
+    if (C % 8 == 0 && ldx % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0)
+      causal_conv8_kernel<<<dim3(T, (C / 8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)x, ldx, w, bias, token_seq, cu_seqlens,
+                                                                            state_slots, state, num_slots, C, N, taps, (bf16_t*)out);
+    else
+      causal_conv_kernel<bf16_t><<<dim3(T, cb), 256, 0, stream>>>((const bf16_t*)x, ldx, w, bias, token_seq, cu_seqlens, state_slots,
+                                                                  state, num_slots, C, N, taps, (bf16_t*)out);
     if (taps > 1)
       conv_history_kernel<bf16_t><<<dim3(B, cb), 256, 0, stream>>>((const bf16_t*)x, ldx, cu_seqlens, state_slots, state, num_slots, C, N, taps);
   } else {

@@ -1078,10 +1078,11 @@ def rope_inplace(x: torch.Tensor, col0: int, heads: int, head_stride: int, rot: 
 
 
 def head_linear(x: torch.Tensor, x_col: int, x_head: int, w: torch.Tensor, heads: int, copy: int = 0,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None, turn: Optional[torch.Tensor] = None) -> torch.Tensor:
     """A product a head: out[t, h, :n_out] = x[t, x_col + h * x_head : .. + n_in] @ w[h] with w [heads, n_in, n_out];
-    the ``copy`` entries behind a head's inputs are handed on behind its outputs.  Returns [T, heads * (n_out + copy)]."""
-    _gpu(x, w, out)
+    the ``copy`` entries behind a head's inputs are handed on behind its outputs, as they are or (``turn``: a table of
+    ``rope_table`` for copy / 2 pairs) turned by the token's angles, neighbours in pairs.  Returns [T, heads * (n_out + copy)]."""
+    _gpu(x, w, out, turn)
     T = x.shape[0]
     if w.dim() != 3 or w.shape[0] != heads or not w.is_contiguous() or w.dtype != x.dtype:
         raise KernelError("head_linear: w must be contiguous [heads, in, out] of the activations' dtype")
@@ -1093,9 +1094,13 @@ def head_linear(x: torch.Tensor, x_col: int, x_head: int, w: torch.Tensor, heads
         out = torch.empty(T, heads * o_head, dtype=x.dtype, device=x.device)
     elif tuple(out.shape) != (T, heads * o_head) or out.dtype != x.dtype or not out.is_contiguous():
         raise KernelError("head_linear: out has the wrong shape or dtype")
+    if turn is not None:
+        if copy % 2 or copy == 0:
+            raise KernelError("head_linear: a part that is turned has an even, positive number of entries")
+        _check_table(turn, T, copy // 2)
     lib = library.core()
     _check(lib, lib.pico_head_linear(_ptr(x), x.stride(0) if T > 1 else x.shape[1], x_col, x_head, _ptr(w), _ptr(out),
-                                     heads * o_head, 0, o_head, _dt(x), T, heads, n_in, n_out, copy, _stream()))
+                                     heads * o_head, 0, o_head, _dt(x), T, heads, n_in, n_out, copy, _ptr(turn), _stream()))
     return out
 
 
@@ -1103,10 +1108,12 @@ def head_linear(x: torch.Tensor, x_col: int, x_head: int, w: torch.Tensor, heads
 SSM_MAX_TAPS, SSM_MAX_STATE = 16, 256
 
 
-def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Tensor, ctx, state: torch.Tensor, n_state: int) -> torch.Tensor:
+def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Tensor, ctx, state: torch.Tensor, n_state: int,
+                single: bool = False) -> torch.Tensor:
     """silu(bias + the causal convolution of the first ``channels`` columns of x with w [channels, taps]) for every
     sequence of the step; inputs before a portion come from the slot's history (``state`` float32
-    [slots, channels, n_state + taps - 1], its last taps - 1 columns), which is brought up to date."""
+    [slots, channels, n_state + taps - 1], its last taps - 1 columns), which is brought up to date.  ``single``: every
+    sequence of the step brings one token (one launch makes the convolution and the history)."""
     _gpu(x, w, bias, state)
     T = x.shape[0]
     taps = w.shape[1]
@@ -1123,7 +1130,7 @@ def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Ten
     lib = library.core()
     _check(lib, lib.pico_causal_conv(_ptr(x), x.stride(0) if T > 1 else x.shape[1], _dt(x), _ptr(w), _ptr(bias), _ptr(ctx.token_seq),
                                      _ptr(ctx.cu_seqlens), _ptr(ctx.state_slots), _ptr(state), state.shape[0], T, B, channels,
-                                     n_state, taps, _ptr(out), _stream()))
+                                     n_state, taps, _ptr(out), 1 if single and T == B else 0, _stream()))
     return out
 
 

@@ -108,10 +108,13 @@ class LatentAttention(Mixer):
     def graph_variant(self, ctx: StepContext) -> tuple:
         return (("latent_attention",) + self.fast.plan(ctx),) if self.fast is not None else ()
 
-    def _per_head(self, x: torch.Tensor, x_head: int, w: torch.Tensor, copy: int = 0) -> torch.Tensor:
-        """out[t, h] = [x[t, h, :in] @ w[h] | x[t, h, in : in + copy]]; x [T, H * x_head]."""
+    def _per_head(self, x: torch.Tensor, x_head: int, w: torch.Tensor, copy: int = 0, turn=None) -> torch.Tensor:
+        """out[t, h] = [x[t, h, :in] @ w[h] | x[t, h, in : in + copy]]; x [T, H * x_head].  ``turn``: the table of the
+        angles by which the copied part is turned on the way (this package's kernel does it in its launch)."""
         T, H = x.shape[0], self.heads
         if x.dtype == torch.bfloat16 and T >= self.LIBRARY_FROM:
+            if turn is not None:
+                kernels.rope_inplace(x, w.shape[1], H, x_head, copy, turn, halves=False)
             # The library's batched product on operands laid out batch by batch ([H, T, in] and [H, T, out], both made
             # here), and never under the library's tuner: handed the rows' own layout (a head's matrix interleaved
             # with the other heads', the batch stride smaller than the row stride) the tuner's copies of the operands
@@ -126,7 +129,7 @@ class LatentAttention(Mixer):
             if copy:
                 out[:, :, n_out:] = xv[:, :, n_in:n_in + copy]
             return out.view(T, H * (n_out + copy))
-        return kernels.head_linear(x, 0, x_head, w, H, copy=copy)
+        return kernels.head_linear(x, 0, x_head, w, H, copy=copy, turn=turn)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         return self.o.partial(self.attend(x, ctx, cache))
@@ -139,9 +142,8 @@ class LatentAttention(Mixer):
         cq = kernels.latent_prepare(y, self.q_rank, self.kv_rank, r, self.wq, self.wkv, self.norm_eps, table,
                                     ctx.slot_mapping[cache.group], cache.k, cache.v)
         q = self.uq(cq)                                          # [T, H (d + r)]
-        if r:
-            kernels.rope_inplace(q, d, H, d + r, r, table, halves=False)
-        ql = self._per_head(q, d + r, self.uk_t, copy=r)         # [T, H (kv_rank + r)]: the queries in the latent's space
+        # the queries in the latent's space, their rotated part turned on the way: [T, H (kv_rank + r)]
+        ql = self._per_head(q, d + r, self.uk_t, copy=r, turn=table if r else None)
         bt = ctx.block_tables[cache.group]
         if self.fast is not None and cache.k.dtype == torch.bfloat16:
             ol = self.fast(ql, cache, bt, ctx)

@@ -77,7 +77,7 @@ class SelectiveStateSpace(Mixer):
         """y * silu(z) [T, inner] in front of the output projection."""
         I, N, R = self.inner, self.state, self.dt_rank
         uz = self.in_proj(x)                                                         # [T, u | z]
-        u = kernels.causal_conv(uz, I, self.conv_w, self.conv_b, ctx, cache.state, N)
+        u = kernels.causal_conv(uz, I, self.conv_w, self.conv_b, ctx, cache.state, N, single=ctx.all_decode)
         dbc = self.x_proj(u)                                                         # [T, d | B | C]
         dt_pre = self.dt_proj(dbc[:, :R], out_dtype=torch.float32)                   # step sizes stay float32 from here on
         chunked = self.act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= self.CHUNKED_FROM

@@ -373,8 +373,9 @@ def test_latent_attention_pieces_against_the_heads_spelled_out(dtype):
     s = s.masked_fill(~(pos[None, :] <= pos[:, None])[None], float("-inf"))
     want = torch.einsum("hij,jhd->ihd", torch.softmax(s, -1), (c_s @ uv.double().T).view(n, H, dv)).reshape(n, -1)
     qg = q.to(DEV).clone()
+    ql = kernels.head_linear(qg, 0, d + r, uk.to(DEV).view(H, d, R).contiguous(), H, copy=r, turn=table)     # turned on the way
     kernels.rope_inplace(qg, d, H, d + r, r, table, False)
-    ql = kernels.head_linear(qg, 0, d + r, uk.to(DEV).view(H, d, R).contiguous(), H, copy=r)
+    assert torch.equal(ql, kernels.head_linear(qg, 0, d + r, uk.to(DEV).view(H, d, R).contiguous(), H, copy=r))   # or beforehand
     bt = torch.tensor([order], dtype=torch.int32, device=DEV)
     ol = kernels.attn_bias_plain(ql, kc, vc, bt, pos.int().to(DEV), torch.zeros(n, dtype=torch.int32, device=DEV), H, 1, R + r, R, m["scale"], 0)
     got = kernels.head_linear(ol, 0, R, uv.to(DEV).view(H, dv, R).transpose(1, 2).contiguous(), H)
