@@ -1,7 +1,8 @@
 // A selective state-space mixer: a short causal convolution per channel and a recurrence whose decay, input and
 // output weights depend on the token.
 //
-//   xc[t][c] = silu(bias[c] + sum_j w[c][j] * x[t - (taps - 1) + j][c])          zeros before a sequence's start
+//   xc[t][c] = silu(bias[c] + sum_j w[j][c] * x[t - (taps - 1) + j][c])          zeros before a sequence's start; w is kept
+//                                                                            tap by tap, [taps, C]: neighbours read neighbours
 //   dt[t][c] = softplus(dtp[t][c] + dt_bias[c]),   A[c][n] = -exp(A_log[c][n])
 //   S[c][n] <- exp(dt A) S + dt xc[t][c] B[t][n];   y[t][c] = sum_n S[c][n] C[t][n] + D[c] xc[t][c]
 //   out[t][c] = y[t][c] * silu(z[t][c])
@@ -36,7 +37,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
   for (int j = 0; j < taps; j++) {
     const int src = t - (taps - 1) + j;                 // token index of this tap's input
     const float v = src >= first ? load_f32(x + (size_t)src * ldx + c) : hist[(taps - 1) + (src - first)];
-    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    acc = fmaf(w[(size_t)j * C + c], v, acc);
   }
   store_f32(out + (size_t)t * C + c, silu_f(acc));
 }
@@ -68,8 +69,9 @@ __global__ __launch_bounds__(256) void causal_conv8_kernel(const bf16_t* __restr
 #pragma unroll
       for (int i = 0; i < 8; i++) v[i] = state[((size_t)slot * C + c0 + i) * (N + taps - 1) + N + (taps - 1) + (src - first)];
     }
-#pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] = fmaf(w[(size_t)(c0 + i) * taps + j], v[i], acc[i]);
+    const float4 w0 = *reinterpret_cast<const float4*>(w + (size_t)j * C + c0), w1 = *reinterpret_cast<const float4*>(w + (size_t)j * C + c0 + 4);
+    acc[0] = fmaf(w0.x, v[0], acc[0]); acc[1] = fmaf(w0.y, v[1], acc[1]); acc[2] = fmaf(w0.z, v[2], acc[2]); acc[3] = fmaf(w0.w, v[3], acc[3]);
+    acc[4] = fmaf(w1.x, v[4], acc[4]); acc[5] = fmaf(w1.y, v[5], acc[5]); acc[6] = fmaf(w1.z, v[6], acc[6]); acc[7] = fmaf(w1.w, v[7], acc[7]);
   }
   uint4 o;
   o.x = pack2_bf16(silu_f(acc[0]), silu_f(acc[1]));
@@ -114,9 +116,9 @@ __global__ __launch_bounds__(256) void causal_conv_step_kernel(const T* __restri
   float keep[SSM_MAX_TAPS];
   for (int j = 0; j < taps - 1; j++) {
     keep[j] = hist[j];
-    acc = fmaf(w[(size_t)c * taps + j], keep[j], acc);
+    acc = fmaf(w[(size_t)j * C + c], keep[j], acc);
   }
-  acc = fmaf(w[(size_t)c * taps + taps - 1], xv, acc);
+  acc = fmaf(w[(size_t)(taps - 1) * C + c], xv, acc);
   for (int j = 0; j + 1 < taps - 1; j++) hist[j] = keep[j + 1];
   if (taps > 1) hist[taps - 2] = xv;
   store_f32(out + (size_t)t * C + c, silu_f(acc));
@@ -149,7 +151,7 @@ extern "C" int pico_causal_conv(const void* x, int ldx, int dtype, const float* 
     if (taps > 1)
       conv_history_kernel<float><<<dim3(B, cb), 256, 0, stream>>>((const float*)x, ldx, cu_seqlens, state_slots, state, num_slots, C, N, taps);
   } else if (dtype == PICO_DTYPE_BF16) {
-    if (C % 8 == 0 && ldx % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0)
+    if (C % 8 == 0 && ldx % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)w % 16 == 0)
       causal_conv8_kernel<<<dim3(T, (C / 8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)x, ldx, w, bias, token_seq, cu_seqlens,
                                                                             state_slots, state, num_slots, C, N, taps, (bf16_t*)out);
     else

@@ -1110,17 +1110,18 @@ SSM_MAX_TAPS, SSM_MAX_STATE = 16, 256
 
 def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Tensor, ctx, state: torch.Tensor, n_state: int,
                 single: bool = False) -> torch.Tensor:
-    """silu(bias + the causal convolution of the first ``channels`` columns of x with w [channels, taps]) for every
+    """silu(bias + the causal convolution of the first ``channels`` columns of x with w [taps, channels] (tap by tap,
+    the last row the current token's)) for every
     sequence of the step; inputs before a portion come from the slot's history (``state`` float32
     [slots, channels, n_state + taps - 1], its last taps - 1 columns), which is brought up to date.  ``single``: every
     sequence of the step brings one token (one launch makes the convolution and the history)."""
     _gpu(x, w, bias, state)
     T = x.shape[0]
-    taps = w.shape[1]
+    taps = w.shape[0]
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < channels:
         raise KernelError("causal_conv: the rows do not hold the channels")
-    if w.dtype != torch.float32 or tuple(w.shape) != (channels, taps) or not w.is_contiguous() or not 1 <= taps <= SSM_MAX_TAPS:
-        raise KernelError(f"causal_conv: the taps are contiguous float32 [{channels}, 1 to {SSM_MAX_TAPS}]")
+    if w.dtype != torch.float32 or tuple(w.shape) != (taps, channels) or not w.is_contiguous() or not 1 <= taps <= SSM_MAX_TAPS:
+        raise KernelError(f"causal_conv: the taps are contiguous float32 [1 to {SSM_MAX_TAPS}, {channels}]")
     _vec(bias, channels, "the convolution's bias")
     if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (channels, n_state + taps - 1) or not state.is_contiguous():
         raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {channels}, {n_state + taps - 1}]")

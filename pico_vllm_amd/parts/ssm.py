@@ -68,7 +68,8 @@ class SelectiveStateSpace(Mixer):
         self.in_proj, self.x_proj = Linear(tensors[n["in"]].to(device)), Linear(tensors[n["x"]].to(device))
         self.dt_proj, self.o = Linear(tensors[n["dt"]].to(device)), Linear(tensors[n["o"]].to(device))
         f32 = lambda k: tensors[n[k]].to(device=device, dtype=torch.float32).contiguous()
-        self.conv_w, self.conv_b, self.dt_bias, self.a_log, self.d = f32("conv"), f32("conv_bias"), f32("dt_bias"), f32("a_log"), f32("d")
+        self.conv_w = f32("conv").t().contiguous()          # tap by tap, [taps, inner]: neighbouring channels side by side
+        self.conv_b, self.dt_bias, self.a_log, self.d = f32("conv_bias"), f32("dt_bias"), f32("a_log"), f32("d")
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         return self.o.partial(self.mix(x, ctx, cache))

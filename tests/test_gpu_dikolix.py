@@ -259,7 +259,7 @@ def test_convolution_and_recurrence_in_portions_and_token_by_token(dtype, C, N, 
             ctx = step_ctx([step[b] for b in live], [fed[b] for b in live], [slots[b] for b in live])
             cat = lambda k: dev(torch.cat([seqs[b][k][fed[b]:fed[b] + step[b]] for b in live]))
             uz, dbc, dtp = cat("uz"), cat("dbc"), cat("dtp")
-            u = kernels.causal_conv(uz, C, dev(w), dev(cb), ctx, state, N)
+            u = kernels.causal_conv(uz, C, dev(w.t()), dev(cb), ctx, state, N, single=all(n == 1 for n in step if n))
             y = kernels.selective_scan(u, dtp, dev(dtb), dbc, R, R + N, dev(a_log), dev(D), uz[:, C:], ctx, state, taps - 1, chunk=chunk)
             at = 0
             for b in live:
