@@ -61,7 +61,7 @@ CONFIGS = {
         (retention(4, 64, 64, [0.97, 0.99, 0.999, 1.0], rot_dims=32, base=500000.0), moe(6, 3, 64, shared=64)),
         (latent(4, 32, 32, 32, 64, 96, base=250000.0, scaling={"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}), moe(8, 2, 32)),
         (ssm(256, 16, 4, 8), moe(4, 1, 64, shared=32)),
-        (latent(8, 16, 16, 48, 96, 48, scale=0.2), moe(6, 3, 64, shared=64))], eps=1e-6, mult=0.8, bigram=(251, 31, 17), loop=(1, 3, 2)),
+        (latent(8, 16, 16, 48, 96, 48, scale=0.2), moe(6, 3, 64, shared=64))], eps=1e-6, mult=0.8, bigram=(251, 29, 13), loop=(1, 3, 2)),
     # no pair table, no loop, no multiplier, one head, a state wider than a wave (two elements a lane), two taps,
     # retention without rotation, one expert a token
     "c": config(130, 96, [
