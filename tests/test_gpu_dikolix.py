@@ -592,3 +592,66 @@ def test_configurations_drawn_at_random_in_mixed_batches(seed):
     for dtype in ("float32", "bfloat16"):
         rows, _ = replay(d, dtype, steps, peak, page, max_live=3)
         compare(name, dtype, rows, reqs, cfg=cfg, tensors=t)
+
+
+def draw_larger_config(seed):
+    """Sizes the matrix-core kernels take (latents and rotated parts in multiples of 32 and 16, widths of 128 to 384, up
+    to 24 experts), every mixer at least once, a loop more often than not."""
+    rng = random.Random(5000 + seed)
+    width = rng.choice([128, 192, 256, 384])
+    kinds = ["latent", "ssm", "retention"] + [rng.choice(["latent", "ssm", "retention"]) for _ in range(rng.randint(0, 2))]
+    rng.shuffle(kinds)
+    layers = []
+    for kind in kinds:
+        if kind == "latent":
+            rot = rng.choice([32, 64])
+            kv = rng.choice([32, 64, 96, 160, 224])
+            mx = latent(rng.choice([2, 4, 5, 8, 16]), rng.choice([16, 32, 64]), rot, rng.choice([16, 32, 64]), rng.choice([64, 96, 192]), kv,
+                        scale=rng.choice([0.08, 0.15]), base=rng.choice([10000.0, 500000.0]),
+                        scaling=rng.choice([None, {"factor": 4.0, "original": 128, "fast": 16.0, "slow": 1.0}]))
+        elif kind == "ssm":
+            mx = ssm(rng.choice([256, 384, 512]), rng.choice([8, 16, 32, 64]), rng.choice([2, 4]), rng.choice([8, 16, 24]))
+        else:
+            H, dk = rng.choice([2, 4, 6]), rng.choice([32, 64, 128])
+            mx = retention(H, dk, rng.choice([32, 64, 128]), [1.0 - 2.0 ** -rng.randint(3, 11) for _ in range(H)],
+                           rot_dims=rng.choice([None, dk, dk // 2]), base=rng.choice([10000.0, 1e6]))
+        E = rng.choice([4, 8, 16, 24])
+        layers.append((mx, moe(E, rng.randint(1, 4), rng.choice([32, 64, 128]), shared=rng.choice([None, 64, 128]))))
+    n = len(layers)
+    start = rng.randint(0, n - 2)
+    loop = rng.choice([None, (start, rng.randint(start + 1, n), 2), (start, rng.randint(start + 1, n), 3)])
+    return config(rng.choice([300, 512]), width, layers, mult=rng.choice([0.5, 0.7, 1.0]), bigram=(rng.choice([509, 4093]), rng.randint(1, 99), rng.randint(1, 99)),
+                  loop=loop), rng.choice([16, 32, 64])
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_larger_configurations_drawn_at_random_with_long_requests(seed):
+    """Requests of up to 500 tokens in portions of up to 200 beside one another (steps of more than 128 tokens, whose
+    recurrences the bfloat16 engine cuts into chunks that run side by side, several sequences a step) and single tokens."""
+    cfg, page = draw_larger_config(seed)
+    t = P.random_model(cfg, 100 + seed)
+    d = write_model(cfg, t, f"dikolix_large{seed}_")
+    name = f"large{seed}"
+    reqs = requests(cfg["vocab"], [500, 150, 330, 40], seed=seed)
+    rng = random.Random(seed)
+    waiting, live, steps, peak = list(reqs), {}, [], 0
+    sizes = [130, 7, 64, 200, 2]
+    while waiting or live:
+        while waiting and len(live) < 3:
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks, at = reqs[rid], live[rid]
+            last = len(toks) - at <= 6
+            n = 1 if last else min(sizes[rng.randrange(len(sizes))], len(toks) - 6 - at)
+            entries.append((rid, toks[at:at + n], [n - 1] if n > 8 else range(n)))
+            live[rid] = at + n
+            if live[rid] == len(toks):
+                end.append(rid)
+        peak = max(peak, sum(roundup(live[r], page) for r in live))
+        for rid in end:
+            del live[rid]
+        steps.append((entries, end))
+    for dtype in ("float32", "bfloat16"):
+        rows, _ = replay(d, dtype, steps, roundup(peak), page, max_live=3)
+        compare(name, dtype, rows, reqs, cfg=cfg, tensors=t)
