@@ -177,7 +177,7 @@ def dikolix_run_order(cfg: DikolixConfig):
 
 def dikolix_spec(cfg: DikolixConfig) -> ModelSpec:
     norm = PartSpec("layer_norm", {"size": cfg.width, "eps": cfg.norm_eps, "weight_name": "", "bias_name": "b"})
-    layers = []
+    layers, unused = [], []
     for i, l in enumerate(cfg.layers):
         m = l.mixer
         if l.type == "latent_attention":
@@ -194,6 +194,8 @@ def dikolix_spec(cfg: DikolixConfig) -> ModelSpec:
                 "norm_eps": cfg.norm_eps, "rotary_dim": m.rot.dims if m.rot else 0, "base": m.rot.base if m.rot else 10000.0,
                 "scaling": m.rot.scaling if m.rot else None})
         if l.mlp is None:
+            # a checkpoint may still hold the second norm and vector of a layer that has no feed-forward to use them
+            unused += [f"l{i}.norm2", f"l{i}.norm2.b", f"l{i}.ls2"]
             layers.append(LayerSpec(prefix=f"l{i}", block="prenorm_scaled_mixer_only",
                                     slots={"norm1": ("norm1", norm), "mixer": ("mix", mixer)},
                                     block_params={"size": cfg.width, "mult": cfg.residual_mult}))
@@ -213,7 +215,7 @@ def dikolix_spec(cfg: DikolixConfig) -> ModelSpec:
         hidden_size=cfg.width, vocab_size=cfg.vocab, embed_name="embed", layers=layers,
         run_order=[RunEntry(i, add_input=again) for i, again in dikolix_run_order(cfg)],
         final_norm=norm, final_norm_name="final.norm", head_name=None, eos_token_id=cfg.eos_token_id,
-        before_layers=before)
+        before_layers=before, ignored_tensors=tuple(unused))
 
 
 def dikolix_sizes(cfg: DikolixConfig) -> dict:

@@ -121,3 +121,17 @@ def test_state_of_parts_around_the_layers_joins_the_cache_manager():
     assert specs[1].kind == "paged_kv" and specs[3] == specs[1] and specs[2] == specs[4] and specs[2].kind == "state"
     m = CacheManager(specs, 8, 10, 2)
     assert len(m.groups) == 2 and m.add_request("x") and m.take_fresh_slots() == [m.slot("x")]
+
+
+def test_a_checkpoint_may_hold_the_unused_second_norm_of_a_layer_without_feed_forward():
+    from dikolix_configs import write_model
+    from pico_vllm_amd.config.registry import load_model_description
+    from pico_vllm_amd.parts.model import model_param_specs
+    from pico_vllm_amd.weights.loader import load_checkpoint
+    t = dict(tensors_of("a"))
+    width = CONFIGS["a"]["width"]
+    t["l1.norm2"], t["l1.norm2.b"], t["l1.ls2"] = (torch.ones(width).bfloat16() for _ in range(3))
+    d = write_model(CONFIGS["a"], t, "dikolix_extra_")
+    _, _, spec = load_model_description(d)
+    out = load_checkpoint(d, model_param_specs(spec), torch.float32, optional=spec.ignored_tensors)
+    assert "l1.norm2" not in out and "l1.norm1" in out
