@@ -22,8 +22,10 @@ BOUND = {"float32": 3e-5, "bfloat16": 7e-2}
 # changes reaches every later position through the recurrent layers: those positions are only held to TAINTED_BOUND.
 # (The margin is counted in units of the router logits' spread over a row; what reaches a router after several layer
 # runs in bfloat16 is off by a few percent of its size, and so are the logits.)
-CLOSE_CALL, TAINTED_BOUND = 0.25, 2.5
-FLOAT32_CLOSE, FLOAT32_LOOSE = 0.01, 1e-3
+CLOSE_CALL, TAINTED_BOUND = 0.4, 2.5
+# float32 rounds too: below FLOAT32_FLIP a choice may really turn (then as in bfloat16); below FLOAT32_CLOSE a head norm
+# multiplies a rounding of 1e-7 by hundreds
+FLOAT32_FLIP, FLOAT32_CLOSE, FLOAT32_LOOSE = 1e-4, 0.01, 1e-3
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 PAGE = {"a": 16, "b": 8, "c": 32, "d": 16}
 
@@ -81,7 +83,7 @@ def compare(name, dtype, rows, reqs, bound=None, cfg=None, tensors=None):
         m = margin_upto(name, toks, pos)
         if not (dtype == "bfloat16" and m < CLOSE_CALL):
             errs.append(e)
-        if dtype == "bfloat16" and m < CLOSE_CALL:
+        if (dtype == "bfloat16" and m < CLOSE_CALL) or m < FLOAT32_FLIP:
             assert e <= TAINTED_BOUND, f"{name} {dtype}: {rid} position {pos}: {e:.3g}"
         elif dtype == "float32" and m < FLOAT32_CLOSE:
             assert e <= FLOAT32_LOOSE, f"{name} {dtype}: {rid} position {pos}: {e:.3g}"
