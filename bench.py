@@ -8,8 +8,9 @@
                                                              continuous batching with prompts cut into portions)
 
   python bench.py --workload designs --layers 4             (Lerazen and Nasedra, each beside the Qwen2.5 shape of equal size,
-                                                             at two sizes: decode at batch 1 and 8, the 2,048-token
-                                                             prefill; --designs nasedra measures that design's pairs only)
+                                                             and Dikolix beside Nasedra, at two sizes: decode at batch 1
+                                                             and 8, the 2,048-token prefill; --designs nasedra measures
+                                                             that design's pairs only)
 
   python bench.py --workload long --shape 32b --device-weights --context 32768
                                                             (one 16k-token prompt in portions of 2,048, then decode at

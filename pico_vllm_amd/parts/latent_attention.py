@@ -61,11 +61,6 @@ class LatentAttention(Mixer):
         self.wq = self.wkv = None
         self.fast = None
 
-    # the attention kernels see values of the latent's size
-    @property
-    def attn_dv(self) -> int:
-        return self.kv_rank
-
     def cache_spec(self) -> CacheSpec:
         return CacheSpec("paged_kv", page_tensors=(PageTensor("k", (1, "page", self.kv_rank + self.r)),
                                                    PageTensor("v", (1, self.kv_rank, "page"))))
