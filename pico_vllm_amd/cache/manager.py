@@ -67,7 +67,8 @@ class CacheManager:
         self.groups: List[CacheGroup] = []
         self.layer_group: Dict[int, int] = {}
         self.state_layers: List[int] = []
-        for layer in sorted(layer_specs):
+        # cache ids are run entries (ints) or, for the parts of a mixer with several caches, tuples that start with one
+        for layer in sorted(layer_specs, key=lambda i: i if isinstance(i, tuple) else (i,)):
             spec = layer_specs[layer]
             if spec.kind == "paged_kv":
                 for gi, g in enumerate(self.groups):
@@ -136,14 +137,19 @@ class CacheManager:
     def advance(self, req: Hashable, num_computed: int) -> None:
         """Record that positions [0, num_computed) are cached, and give back
         the pages that every window has passed: the next query sits at
-        position num_computed or later and reads keys > position - window.  Pages that
+        position num_computed or later and reads keys > position - window (or, in a group whose
+        positions read their own chunk only, keys from the start of its chunk).  Pages that
         hold any of a group's first ``keep_first`` positions are never given back early."""
         rc = self.requests[req]
         rc.num_computed = num_computed
         for gi, g in enumerate(self.groups):
-            if g.window <= 0:
+            if g.window > 0:
+                first_needed = num_computed - g.window + 1      # lowest key position still readable
+            elif g.spec.chunk > 0:
+                # the next query's chunk starts here or later, and it reads nothing in front of its chunk
+                first_needed = num_computed // g.spec.chunk * g.spec.chunk
+            else:
                 continue
-            first_needed = num_computed - g.window + 1      # lowest key position still readable
             if first_needed <= 0:
                 continue
             dead_upto = min(first_needed // self.page_size, len(rc.tables[gi]))

@@ -72,8 +72,15 @@ class CacheStorage:
             else:
                 self._layers[layer] = None
 
-    def layer(self, index: int, read_only: bool = False):
-        """The cache of run entry ``index``; ``read_only`` for a run that was given another run's cache."""
+    def layer(self, index, read_only: bool = False):
+        """The cache of run entry ``index``; ``read_only`` for a run that was given another run's cache.  A mixer that
+        keeps several caches gets a list of them, in the order of its spec's parts (nested like the spec)."""
+        if index not in self._layers:
+            head = index if isinstance(index, tuple) else (index,)
+            n = len(head)
+            kids = sorted({k[n] for k in self._layers if isinstance(k, tuple) and len(k) > n and k[:n] == head})
+            if kids:
+                return [self.layer(head + (j,), read_only) for j in kids]
         entry = self._layers.get(index)
         if read_only and isinstance(entry, PagedKVLayer):
             return PagedKVLayer(entry.tensors, entry.group, entry.page_size, read_only=True)

@@ -9,6 +9,9 @@
 //   visible to every later query (at their true distance); optionally o_i is multiplied element by element with
 //   sigmoid(gate_i) before it is written
 //   softmax over the visible keys, o_i = sum_j p_ij v_j
+//   instead of a window, chunks: key j <= i is seen iff floor(i / chunk) == floor(j / chunk), chunks counted from
+//   position 0; optionally a sink (a key of score 0 without a value: the softmax's denominator gains a 1); the gate may be
+//   one number a head; several kv heads (of keys) may share one head of values (v_div of them each)
 //
 // A page holds k as [kv heads, page, dk] and v as [kv heads, dv, page].  Scores, softmax and the sums over keys are
 // float32 whatever the storage type.  This file holds the plain kernel (one wave per query token and head, any sizes,
@@ -20,6 +23,10 @@ struct BiasParams {
   int temp_every, window;
   float softcap;      // 0: none
   int keep_first;     // with a window: keys below this position are seen whatever their distance
+  int chunk;          // > 0: position i sees key j <= i only if floor(i / chunk) == floor(j / chunk) (instead of a window)
+  int sink;           // != 0: one more key of score 0 and no value, p_j = exp(s_j) / (1 + sum exp(s))
+  int gate_heads;     // != 0: the gate holds one number a head (gate[t][h]) instead of one an output element
+  int v_div;          // kv head g's values are value head g / v_div (several kv heads of keys over one head of values)
 };
 
 __device__ __forceinline__ float query_scale(const BiasParams& p, int pos) {
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, int max_pages, const int* __restrict__ positions,
     const int* __restrict__ token_seq, T* __restrict__ out, int nq, int nkv, int dk, int dv, int P, BiasParams bp,
-    int num_pages, const T* __restrict__ gate, int gate_stride) {
+    int num_pages, const T* __restrict__ gate, int gate_stride, float* __restrict__ out32) {
   extern __shared__ float lds[];
   float* qs = lds;        // [dk]
   float* ps = lds + dk;   // [64]
@@ -104,7 +111,8 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
   const int g = h / (nq / nkv);
   const int pos = positions[t];
   const int* bt = block_table + (size_t)token_seq[t] * max_pages;
-  const int lo = bp.window > 0 ? max(0, pos - bp.window + 1) : 0;
+  const int lo = bp.chunk > 0 ? pos / bp.chunk * bp.chunk : bp.window > 0 ? max(0, pos - bp.window + 1) : 0;
+  const int gv = g / bp.v_div, nv = nkv / bp.v_div;        // the head of values, and how many there are
   const float qscale = query_scale(bp, pos), slope = head_slope(bp, h, nq);
   const T* qrow = q + (size_t)t * q_stride + (size_t)h * dk;
   for (int j = lane; j < dk; j += 64) qs[j] = load_f32(qrow + j);
@@ -149,7 +157,7 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
       if (kpos < lo && kpos >= keep) continue;
       int page = bt[kpos / P];
       page = min(max(page, 0), num_pages - 1);
-      const T* vp = v_cache + ((size_t)page * nkv + g) * dv * P + kpos % P;
+      const T* vp = v_cache + ((size_t)page * nv + gv) * dv * P + kpos % P;
       const float pk = ps[kk];
 #pragma unroll
       for (int i = 0; i < NV; i++) {
@@ -161,14 +169,16 @@ __global__ __launch_bounds__(64) void attn_bias_plain_kernel(
     for (int i = 0; i < NV; i++) acc[i] = fmaf(acc[i], alpha, blk[i]);
     m = m_new;
   }
+  if (bp.sink) l += expf(-m);                              // the sink's exp(0 - m); the query's own key is always seen
   T* o = out + ((size_t)t * nq + h) * dv;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int dim = lane + 64 * i;
     if (dim >= dv) continue;
     float v = acc[i] / l;
-    if (gate) v *= 1.0f / (1.0f + expf(-load_f32(gate + (size_t)t * gate_stride + (size_t)h * dv + dim)));
-    store_f32(o + dim, v);
+    if (gate) v *= 1.0f / (1.0f + expf(-load_f32(gate + (size_t)t * gate_stride + (bp.gate_heads ? (size_t)h : (size_t)h * dv + dim))));
+    if (out32) out32[((size_t)t * nq + h) * dv + dim] = v;
+    else store_f32(o + dim, v);
   }
 }
 
@@ -176,8 +186,8 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
                                     const int* block_table, int max_pages, const int* positions, const int* token_seq,
                                     void* out, int T, int nq, int nkv, int dk, int dv, int P, int window, float scale,
                                     float temp_coef, int temp_every, float slope_span, int num_pages,
-                                    float softcap, int keep_first, const void* gate, int gate_stride,
-                                    hipStream_t stream) {
+                                    float softcap, int keep_first, const void* gate, int gate_stride, int chunk, int sink,
+                                    int gate_heads, int v_div, int out_f32, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && dk > 0 && dv > 0 && P > 0 && max_pages > 0 && num_pages > 0,
                "pico_attn_bias_plain: bad sizes");
   PICO_REQUIRE(nq % nkv == 0, "pico_attn_bias_plain: %d query heads are not a multiple of %d kv heads", nq, nkv);
@@ -186,30 +196,33 @@ extern "C" int pico_attn_bias_plain(const void* q, int q_stride, int dtype, cons
   PICO_REQUIRE(q_stride >= nq * dk, "pico_attn_bias_plain: query row stride too small");
   PICO_REQUIRE(window >= 0 && temp_every >= 0 && slope_span >= 0.f, "pico_attn_bias_plain: window, interval and span must not be negative");
   PICO_REQUIRE(softcap >= 0.f && keep_first >= 0, "pico_attn_bias_plain: cap and kept first positions must not be negative");
-  PICO_REQUIRE(gate == nullptr || gate_stride >= nq * dv, "pico_attn_bias_plain: gate row stride too small");
+  PICO_REQUIRE(gate == nullptr || gate_stride >= (gate_heads ? nq : nq * dv), "pico_attn_bias_plain: gate row stride too small");
+  PICO_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "pico_attn_bias_plain: chunks or a window, not both");
+  PICO_REQUIRE(v_div >= 1 && nkv % v_div == 0, "pico_attn_bias_plain: %d kv heads do not share values %d each", nkv, v_div);
   if (T == 0) return 0;
-  const BiasParams bp{scale, temp_coef, slope_span, temp_every, window, softcap, keep_first};
+  const BiasParams bp{scale, temp_coef, slope_span, temp_every, window, softcap, keep_first, chunk, sink, gate_heads, v_div};
+  float* out32 = out_f32 ? (float*)out : nullptr;
   dim3 grid(T, nq);
   const size_t lds = (size_t)(dk + 64) * sizeof(float);
   if (dtype == PICO_DTYPE_F32) {
     if (dv <= 256)
       attn_bias_plain_kernel<float, 4><<<grid, 64, lds, stream>>>(
           (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
-          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
+          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride, out32);
     else
       attn_bias_plain_kernel<float, 8><<<grid, 64, lds, stream>>>(
           (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_pages, positions,
-          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride);
+          token_seq, (float*)out, nq, nkv, dk, dv, P, bp, num_pages, (const float*)gate, gate_stride, out32);
   }
   else if (dtype == PICO_DTYPE_BF16) {
     if (dv <= 256)
       attn_bias_plain_kernel<bf16_t, 4><<<grid, 64, lds, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
-          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
+          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride, out32);
     else
       attn_bias_plain_kernel<bf16_t, 8><<<grid, 64, lds, stream>>>(
           (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, positions,
-          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride);
+          token_seq, (bf16_t*)out, nq, nkv, dk, dv, P, bp, num_pages, (const bf16_t*)gate, gate_stride, out32);
   }
   else
     PICO_REQUIRE(false, "pico_attn_bias_plain: unknown dtype %d", dtype);

@@ -53,6 +53,10 @@ struct BiasArgs {
   int keep_first;
   const bf16_t* gate;
   int gate_stride;
+  // chunk > 0 (instead of a window): key j <= i is seen iff floor(i / chunk) == floor(j / chunk); sink: the softmax's
+  // denominator gains exp(0) (a key of score 0 without a value); gate_heads: the gate holds one number a head;
+  // v_div: kv head g reads value head g / v_div; out_f32: `out` is float32
+  int chunk, sink, gate_heads, v_div, out_f32;
 };
 
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + __expf(-x)); }
@@ -91,8 +95,9 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
   const int p0 = found ? a.positions[t0] : 0;           // the block's first position; its tokens follow one another
   const int my_pos = p0 + (col_ok ? my_tok : 0);
   const int hi = p0 + ntok;                             // keys below hi are read
-  const int lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
-  const int my_lo = a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
+  const int lo = a.chunk > 0 ? p0 / a.chunk * a.chunk : a.window > 0 ? max(0, p0 - a.window + 1) : 0;
+  const int my_lo = a.chunk > 0 ? my_pos / a.chunk * a.chunk : a.window > 0 ? max(0, my_pos - a.window + 1) : 0;
+  const int gv = g / a.v_div, nv = a.nkv / a.v_div;      // the head of values, and how many there are
   const int keep = a.window > 0 ? a.keep_first : 0;     // keys below are seen although a window has passed them
   const float inv_cap = a.softcap > 0.f ? 1.0f / a.softcap : 0.f;
   const int* bt = a.block_table + (size_t)b * a.max_pages;
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
       {
         const int pos = min(key0 + 8 * kq, last_group);
         const int page = min(max(bt[pos >> pshift], 0), a.num_pages - 1);
-        const bf16_t* vp = a.v_cache + ((((size_t)page * a.nkv + g) * DV + col) << pshift) + (pos & (a.P - 1));
+        const bf16_t* vp = a.v_cache + ((((size_t)page * nv + gv) * DV + col) << pshift) + (pos & (a.P - 1));
 #pragma unroll
         for (int tt = 0; tt < DT; tt++) vr[tt] = *reinterpret_cast<const uint4*>(vp + ((size_t)tt * 16 << pshift));
       }
@@ -261,12 +266,19 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
     if (kq == 0) { a.parts_ml[2 * c] = M_all; a.parts_ml[2 * c + 1] = L; }
     return;
   }
-  const float inv = 1.0f / L;
+  if (a.sink) L += __expf(-M_all);                        // the column's own key is always seen: M_all is finite
+  float inv = 1.0f / L;
+  if (a.gate && a.gate_heads) inv *= sigmoid_f32(bf16_to_f32(a.gate[(size_t)t * a.gate_stride + head]));
   bf16_t* orow = a.out + ((size_t)t * a.nq + head) * DV + 4 * kq;
-  const bf16_t* grow = a.gate ? a.gate + (size_t)t * a.gate_stride + (size_t)head * DV + 4 * kq : nullptr;
+  const bf16_t* grow = a.gate && !a.gate_heads ? a.gate + (size_t)t * a.gate_stride + (size_t)head * DV + 4 * kq : nullptr;
 #pragma unroll
   for (int tt = 0; tt < DT; tt++) {
     float g0 = inv, g1 = inv, g2 = inv, g3 = inv;
+    if (a.out_f32) {
+      float* o32 = reinterpret_cast<float*>(a.out) + ((size_t)t * a.nq + head) * DV + 4 * kq + 16 * tt;
+      *reinterpret_cast<f32x4*>(o32) = f32x4{o[tt][0] * g0, o[tt][1] * g1, o[tt][2] * g2, o[tt][3] * g3};
+      continue;
+    }
     if (grow) {
       const uint2 gv = *reinterpret_cast<const uint2*>(grow + 16 * tt);
       g0 *= sigmoid_f32(__uint_as_float(gv.x << 16));
@@ -285,7 +297,7 @@ __global__ __launch_bounds__(256, 2) void attn_bias_kernel(const BiasArgs a) {
 // The pieces of a column's keys put together: out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), z in ascending order.
 __global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bias_merge_kernel(
     const float* __restrict__ parts_o, const float* __restrict__ parts_ml, int chunks, int ncols, bf16_t* __restrict__ out,
-    const bf16_t* __restrict__ gate, int gate_stride, int nq) {
+    const bf16_t* __restrict__ gate, int gate_stride, int nq, int sink, int gate_heads, int out_f32) {
   // the pieces' maxima and sums once into LDS (one load a thread, all in flight together), then every thread its sum
   __shared__ float ms[MAX_PIECES], ws[MAX_PIECES];
   const int c = blockIdx.x, d = threadIdx.x;
@@ -305,9 +317,11 @@ __global__ __launch_bounds__(DV <= 64 ? 64 : DV <= 128 ? 128 : 256) void attn_bi
     L += ws[z] * w;
     acc += parts_o[((size_t)z * ncols + c) * DV + d] * w;
   }
+  if (sink) L += __expf(-M);
   float v = acc / L;
-  if (gate) v *= sigmoid_f32(bf16_to_f32(gate[(size_t)(c / nq) * gate_stride + (size_t)(c % nq) * DV + d]));
-  out[(size_t)c * DV + d] = f32_to_bf16(v);
+  if (gate) v *= sigmoid_f32(bf16_to_f32(gate[(size_t)(c / nq) * gate_stride + (gate_heads ? (size_t)(c % nq) : (size_t)(c % nq) * DV + d)]));
+  if (out_f32) reinterpret_cast<float*>(out)[(size_t)c * DV + d] = v;
+  else out[(size_t)c * DV + d] = f32_to_bf16(v);
 }
 
 // split != 0: one block of 16 columns a workgroup, its keys shared by the four waves; else four blocks a workgroup.
@@ -315,7 +329,8 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
                           int max_pages, const int* cu_seqlens, const int* positions, int num_seqs, int T, void* out,
                           int nq, int nkv, int dk, int dv, int P, int num_pages, float scale, int window, float temp_coef,
                           int temp_every, float slope_span, int split, int chunks, float* parts_o, float* parts_ml,
-                          float softcap, int keep_first, const void* gate, int gate_stride, hipStream_t stream) {
+                          float softcap, int keep_first, const void* gate, int gate_stride, int chunk, int sink,
+                          int gate_heads, int v_div, int out_f32, hipStream_t stream) {
   PICO_REQUIRE(dk == DK && dv == DV, "pico_attnb: built for keys of %d and values of %d, asked for %d and %d", DK, DV, dk, dv);
   PICO_REQUIRE(T >= 0 && num_seqs > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && max_pages > 0 && num_pages > 0,
                "pico_attnb: bad sizes");
@@ -325,8 +340,10 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(chunks >= 1 && chunks <= MAX_PIECES && (chunks == 1 || (split && parts_o && parts_ml)),
                "pico_attnb: pieces of the keys go with one block a workgroup and need room for the parts");
   PICO_REQUIRE(softcap >= 0.f && keep_first >= 0, "pico_attnb: cap and kept first positions must not be negative");
-  PICO_REQUIRE(gate == nullptr || (gate_stride >= nq * DV && gate_stride % 4 == 0 && (uintptr_t)gate % 8 == 0),
+  PICO_REQUIRE(gate == nullptr || (gate_heads ? gate_stride >= nq : (gate_stride >= nq * DV && gate_stride % 4 == 0 && (uintptr_t)gate % 8 == 0)),
                "pico_attnb: gate rows must be 8-byte aligned and hold all heads");
+  PICO_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "pico_attnb: chunks or a window, not both");
+  PICO_REQUIRE(v_div >= 1 && nkv % v_div == 0, "pico_attnb: %d kv heads do not share values %d each", nkv, v_div);
   if (T == 0) return 0;
   const int R = nq / nkv;
   const int tpb = R >= 16 ? 1 : 16 / R, hb = R > 16 ? (R + 15) / 16 : 1;
@@ -335,13 +352,14 @@ extern "C" int pico_attnb(const void* q, int q_stride, const void* k_cache, cons
   PICO_REQUIRE(tiles < (1ll << 30), "pico_attnb: too many blocks");
   BiasArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,
              cu_seqlens, positions, (bf16_t*)out, num_seqs, nq, nkv, P, num_pages, window, temp_every, scale, temp_coef,
-             slope_span, chunks, T * nq, parts_o, parts_ml, softcap, keep_first, (const bf16_t*)gate, gate_stride};
+             slope_span, chunks, T * nq, parts_o, parts_ml, softcap, keep_first, (const bf16_t*)gate, gate_stride,
+             chunk, sink, gate_heads, v_div, out_f32};
   if (split) {
     attn_bias_kernel<true><<<dim3((unsigned)tiles, nkv, chunks), 256, 0, stream>>>(a);
     if (chunks > 1)
       attn_bias_merge_kernel<<<T * nq, DV <= 64 ? 64 : DV <= 128 ? 128 : 256, 0, stream>>>(parts_o, parts_ml, chunks, T * nq,
                                                                                            (bf16_t*)out, (const bf16_t*)gate,
-                                                                                           gate_stride, nq);
+                                                                                           gate_stride, nq, sink, gate_heads, out_f32);
   } else
     attn_bias_kernel<false><<<dim3((unsigned)((tiles + 3) / 4), nkv), 256, 0, stream>>>(a);
   PICO_LAUNCH_CHECK();

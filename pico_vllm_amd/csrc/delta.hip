@@ -1,0 +1,282 @@
+// Recurrent mixers whose state is a matrix S [dk, dv] per head and request, walked token by token:
+//
+//     S <- diag(g_t) S                        (g_t: a decay per key channel, or one per head)
+//     u  = beta_t (v_t - S^T k_t)             (the delta rule; without it u = beta_t v_t)
+//     S <- S + k_t u^T
+//     o_t = S^T q_t                           (the read-out sees the token's own write)
+//
+// The gated delta rule uses it as it stands; a state-space (duality) layer is the same walk without the correction, with
+// k = B, q = C, beta = dt and one decay exp(-a dt) a head.  Query/key heads may be shared by several value heads (head
+// h reads q/k head h / (H / KVH)).  Everything here is float32: the state, the decays, beta, the unit norms; only the
+// values come in the activations' storage type.
+//
+//   pico_delta_prep:   unit vectors q, k per head (x / sqrt(sum x^2 + 1e-6), q times qscale), beta = sigmoid(.),
+//                      g = exp(-exp(A_log_h) softplus(a2 (a1 h) + dt_bias)) per head and key channel
+//   pico_ssd_prep:     dt = softplus(dt_raw + dt_bias), g = exp(-exp(A_log_h) dt) per head; B and C widened to float32
+//   pico_delta_scan:   the walk.  A value channel's column of S does not depend on the other columns, so a wave takes
+//                      64 / KS columns with the key channels of each cut over KS lanes (KPL channels a lane, in
+//                      registers for the whole step); the two sums over key channels meet across those lanes.
+//   pico_gated_group_norm: (y + D_h x) silu(z), RMS-normed in equal parts of the row, times a weight
+#include "common.h"
+
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// grid (T); x: the convolved q | k (columns q_col .., k_col .., KVH heads of dk each); y: the row that holds beta's
+// logits (b_col, H of them) and the low-rank activations (a_col, R of them); a2 [H * dk, R].
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prep_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col,
+                                                         const T* __restrict__ y, int ldy, int b_col, int a_col,
+                                                         const T* __restrict__ a2, const float* __restrict__ dt_bias,
+                                                         const float* __restrict__ a_log, float qscale, float* __restrict__ qn,
+                                                         float* __restrict__ kn, float* __restrict__ g, float* __restrict__ beta,
+                                                         int H, int KVH, int dk, int R) {
+  extern __shared__ float low[];           // [R]
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const T* yr = y + (size_t)t * ldy;
+  for (int r = threadIdx.x; r < R; r += blockDim.x) low[r] = load_f32(yr + a_col + r);
+  __syncthreads();
+  for (int u = wave; u < 2 * KVH; u += nw) {
+    const bool is_q = u < KVH;
+    const int hh = is_q ? u : u - KVH;
+    const T* src = x + (size_t)t * ldx + (is_q ? q_col : k_col) + (size_t)hh * dk;
+    float ss = 0.f;
+    for (int i = lane; i < dk; i += 64) { const float v = load_f32(src + i); ss = fmaf(v, v, ss); }
+    const float r = (is_q ? qscale : 1.0f) / sqrtf(wave_sum(ss) + 1e-6f);
+    float* dst = (is_q ? qn : kn) + ((size_t)t * KVH + hh) * dk;
+    for (int i = lane; i < dk; i += 64) dst[i] = load_f32(src + i) * r;
+  }
+  for (int c = threadIdx.x; c < H * dk; c += blockDim.x) {
+    const T* w = a2 + (size_t)c * R;
+    float z = dt_bias[c];
+    for (int r = 0; r < R; r++) z = fmaf(load_f32(w + r), low[r], z);
+    g[(size_t)t * H * dk + c] = expf(-expf(a_log[c / dk]) * softplus_f(z));
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)t * H + h] = sigmoid_f(load_f32(yr + b_col + h));
+}
+
+extern "C" int pico_delta_prep(const void* x, int ldx, int q_col, int k_col, const void* y, int ldy, int b_col, int a_col,
+                               int dtype, const void* a2, const float* dt_bias, const float* a_log, float qscale, float* qn,
+                               float* kn, float* g, float* beta, int T, int H, int KVH, int dk, int R, hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && dk > 0 && R > 0 && R <= 8192, "pico_delta_prep: bad sizes");
+  PICO_REQUIRE(ldx >= q_col + KVH * dk && ldx >= k_col + KVH * dk && ldy >= b_col + H && ldy >= a_col + R,
+               "pico_delta_prep: the rows do not hold what is read");
+  if (T == 0) return 0;
+  const size_t lds = (size_t)R * sizeof(float);
+  if (dtype == PICO_DTYPE_F32)
+    delta_prep_kernel<float><<<T, 256, lds, stream>>>((const float*)x, ldx, q_col, k_col, (const float*)y, ldy, b_col, a_col,
+                                                      (const float*)a2, dt_bias, a_log, qscale, qn, kn, g, beta, H, KVH, dk, R);
+  else if (dtype == PICO_DTYPE_BF16)
+    delta_prep_kernel<bf16_t><<<T, 256, lds, stream>>>((const bf16_t*)x, ldx, q_col, k_col, (const bf16_t*)y, ldy, b_col, a_col,
+                                                       (const bf16_t*)a2, dt_bias, a_log, qscale, qn, kn, g, beta, H, KVH, dk, R);
+  else
+    PICO_REQUIRE(false, "pico_delta_prep: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// grid (T); bc: the convolved B | C (columns b_col .., c_col .., n each); dt_raw: H columns of y from dt_col.
+template <typename T>
+__global__ __launch_bounds__(256) void ssd_prep_kernel(const T* __restrict__ bc, int ldb, int b_col, int c_col, int n,
+                                                       const T* __restrict__ y, int ldy, int dt_col,
+                                                       const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                                                       float* __restrict__ bf, float* __restrict__ cf, float* __restrict__ g,
+                                                       float* __restrict__ dt, int H) {
+  const int t = blockIdx.x;
+  const T* br = bc + (size_t)t * ldb;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    bf[(size_t)t * n + i] = load_f32(br + b_col + i);
+    cf[(size_t)t * n + i] = load_f32(br + c_col + i);
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    const float d = softplus_f(load_f32(y + (size_t)t * ldy + dt_col + h) + dt_bias[h]);
+    dt[(size_t)t * H + h] = d;
+    g[(size_t)t * H + h] = expf(-expf(a_log[h]) * d);
+  }
+}
+
+extern "C" int pico_ssd_prep(const void* bc, int ldb, int b_col, int c_col, int n, const void* y, int ldy, int dt_col, int dtype,
+                             const float* dt_bias, const float* a_log, float* bf, float* cf, float* g, float* dt, int T, int H,
+                             hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0 && n > 0 && ldb >= b_col + n && ldb >= c_col + n && ldy >= dt_col + H, "pico_ssd_prep: bad sizes");
+  if (T == 0) return 0;
+  if (dtype == PICO_DTYPE_F32)
+    ssd_prep_kernel<float><<<T, 256, 0, stream>>>((const float*)bc, ldb, b_col, c_col, n, (const float*)y, ldy, dt_col, dt_bias,
+                                                  a_log, bf, cf, g, dt, H);
+  else if (dtype == PICO_DTYPE_BF16)
+    ssd_prep_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)bc, ldb, b_col, c_col, n, (const bf16_t*)y, ldy, dt_col, dt_bias,
+                                                   a_log, bf, cf, g, dt, H);
+  else
+    PICO_REQUIRE(false, "pico_ssd_prep: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The walk.  grid (sequences, heads, ceil(dv / VC)), one wave a workgroup; VC = 64 / KS value columns a wave; lane
+// = ks * VC + vc holds S[ks * KPL .. ks * KPL + KPL - 1][v0 + vc].  The sums over key channels are added lane-locally in
+// channel order and then across the KS lanes of a column in a fixed tree: a token's output does not depend on how its
+// sequence was cut into steps or on what else the step holds.
+// ---------------------------------------------------------------------------
+template <typename TV, int KPL, bool DELTA>
+__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                        const TV* __restrict__ v, int ldv, const float* __restrict__ g,
+                                                        int g_channels, const float* __restrict__ beta,
+                                                        const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                                                        float* __restrict__ state, float* __restrict__ out, int H, int KVH,
+                                                        int dk, int dv, int KS, int num_slots) {
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int VC = 64 / KS, vc = lane % VC, ks = lane / VC;
+  const int col = blockIdx.z * VC + vc;
+  const int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1], slot = state_slots[b];
+  if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;
+  const bool col_ok = col < dv;
+  const int cin = min(col, dv - 1);
+  const int c0 = ks * KPL;
+  const int kvh = h / (H / KVH);
+  float* sp = state + (((size_t)slot * H + h) * dk) * dv + cin;
+  float S[KPL];
+#pragma unroll
+  for (int i = 0; i < KPL; i++) S[i] = (c0 + i < dk) ? sp[(size_t)(c0 + i) * dv] : 0.f;
+  float kk[KPL], qq[KPL], gg[KPL], vv, bb;
+  auto fetch = [&](int t) {
+    const float* kr = k + ((size_t)t * KVH + kvh) * dk;
+    const float* qr = q + ((size_t)t * KVH + kvh) * dk;
+#pragma unroll
+    for (int i = 0; i < KPL; i++) {
+      const int c = min(c0 + i, dk - 1);
+      kk[i] = kr[c];
+      qq[i] = qr[c];
+      gg[i] = g_channels ? g[((size_t)t * H + h) * dk + c] : 0.f;
+    }
+    if (!g_channels) {
+      const float gh = g[(size_t)t * H + h];
+#pragma unroll
+      for (int i = 0; i < KPL; i++) gg[i] = gh;
+    }
+#pragma unroll
+    for (int i = 0; i < KPL; i++)
+      if (c0 + i >= dk) { kk[i] = 0.f; qq[i] = 0.f; gg[i] = 1.f; }
+    vv = load_f32(v + (size_t)t * ldv + (size_t)h * dv + cin);
+    bb = beta[(size_t)t * H + h];
+  };
+  fetch(t_begin);
+  for (int t = t_begin; t < t_end; t++) {
+    float kc[KPL], qc[KPL], gc[KPL];
+#pragma unroll
+    for (int i = 0; i < KPL; i++) { kc[i] = kk[i]; qc[i] = qq[i]; gc[i] = gg[i]; }
+    const float vt = vv, bt = bb;
+    if (t + 1 < t_end) fetch(t + 1);                     // the next token's operands travel while this one is worked on
+    float u = bt * vt;
+    if (DELTA) {
+      float sk = 0.f;
+#pragma unroll
+      for (int i = 0; i < KPL; i++) {
+        S[i] *= gc[i];
+        sk = fmaf(S[i], kc[i], sk);
+      }
+      for (int o = VC; o < 64; o <<= 1) sk += __shfl_xor(sk, o);
+      u = bt * (vt - sk);
+    } else {
+#pragma unroll
+      for (int i = 0; i < KPL; i++) S[i] *= gc[i];
+    }
+    float so = 0.f;
+#pragma unroll
+    for (int i = 0; i < KPL; i++) {
+      S[i] = fmaf(kc[i], u, S[i]);
+      so = fmaf(S[i], qc[i], so);
+    }
+    for (int o = VC; o < 64; o <<= 1) so += __shfl_xor(so, o);
+    if (ks == 0 && col_ok) out[((size_t)t * H + h) * dv + col] = so;
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int i = 0; i < KPL; i++)
+      if (c0 + i < dk) sp[(size_t)(c0 + i) * dv] = S[i];
+  }
+}
+
+#define DELTA_MAX_KEY_DIM 512
+
+extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, int ldv, int v_dtype, const float* g,
+                               int g_channels, const float* beta, const int* cu_seqlens, const int* state_slots, float* state,
+                               float* out, int num_seqs, int H, int KVH, int dk, int dv, int num_slots, int delta,
+                               hipStream_t stream) {
+  PICO_REQUIRE(num_seqs >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && dk > 0 && dk <= DELTA_MAX_KEY_DIM && dv > 0 && num_slots > 0,
+               "pico_delta_scan: bad sizes (at most %d key channels a head)", DELTA_MAX_KEY_DIM);
+  PICO_REQUIRE(ldv >= H * dv && H <= 65535, "pico_delta_scan: the rows do not hold the values");
+  if (num_seqs == 0) return 0;
+  // key channels a lane: the fewest of 4, 8, 16, 32 with which at most 4 lanes share a column; beyond 128 channels
+  // more lanes a column
+  int kpl = 4;
+  while (kpl < 32 && 4 * kpl < dk) kpl *= 2;
+  int KS = 1;
+  while (KS * kpl < dk) KS *= 2;
+  const int VC = 64 / KS;
+  const dim3 grid(num_seqs, H, (dv + VC - 1) / VC);
+  PICO_REQUIRE(grid.z <= 65535, "pico_delta_scan: too many value channels");
+#define GO(TV, KPL)                                                                                                         \
+  do {                                                                                                                      \
+    if (delta)                                                                                                              \
+      delta_scan_kernel<TV, KPL, true><<<grid, 64, 0, stream>>>(q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens,    \
+                                                                state_slots, state, out, H, KVH, dk, dv, KS, num_slots);    \
+    else                                                                                                                    \
+      delta_scan_kernel<TV, KPL, false><<<grid, 64, 0, stream>>>(q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens,   \
+                                                                 state_slots, state, out, H, KVH, dk, dv, KS, num_slots);   \
+  } while (0)
+#define PICK(TV)                    \
+  do {                              \
+    if (kpl == 4) GO(TV, 4);        \
+    else if (kpl == 8) GO(TV, 8);   \
+    else if (kpl == 16) GO(TV, 16); \
+    else GO(TV, 32);                \
+  } while (0)
+  if (v_dtype == PICO_DTYPE_F32) PICK(float);
+  else if (v_dtype == PICO_DTYPE_BF16) PICK(bf16_t);
+  else PICO_REQUIRE(false, "pico_delta_scan: unknown dtype %d", v_dtype);
+#undef PICK
+#undef GO
+  PICO_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[t] = norm_groups( (y[t] + D_h x[t]) * silu(z[t]) ) * w: the row of H * dv entries is cut into `groups` equal parts,
+// each over its own root mean square.  grid (T, groups); y float32 [T, H * dv]; x, z columns of wider rows.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ x, int ldx,
+                                                               const T* __restrict__ z, int ldz, const float* __restrict__ D,
+                                                               const float* __restrict__ w, float eps, T* __restrict__ out,
+                                                               int H, int dv, int groups) {
+  extern __shared__ float part[];
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, gi = blockIdx.y, n = H * dv / groups, base = gi * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int c = base + i;
+    const float zz = load_f32(z + (size_t)t * ldz + c);
+    const float val = fmaf(D[c / dv], load_f32(x + (size_t)t * ldx + c), y[(size_t)t * H * dv + c]) * (zz / (1.0f + expf(-zz)));
+    part[i] = val;
+    ss = fmaf(val, val, ss);
+  }
+  const float r = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) store_f32(out + (size_t)t * H * dv + base + i, part[i] * r * w[base + i]);
+}
+
+extern "C" int pico_gated_group_norm(const float* y, const void* x, int ldx, const void* z, int ldz, int dtype, const float* D,
+                                     const float* w, float eps, void* out, int T, int H, int dv, int groups,
+                                     hipStream_t stream) {
+  PICO_REQUIRE(T >= 0 && H > 0 && dv > 0 && groups > 0 && (H * dv) % groups == 0 && groups <= 65535, "pico_gated_group_norm: bad sizes");
+  PICO_REQUIRE(H * dv / groups <= 16384 && ldx >= H * dv && ldz >= H * dv, "pico_gated_group_norm: a part of at most 16384 entries");
+  if (T == 0) return 0;
+  const size_t lds = (size_t)(H * dv / groups) * sizeof(float);
+  const dim3 grid(T, groups);
+  if (dtype == PICO_DTYPE_F32)
+    gated_group_norm_kernel<float><<<grid, 256, lds, stream>>>(y, (const float*)x, ldx, (const float*)z, ldz, D, w, eps, (float*)out, H, dv, groups);
+  else if (dtype == PICO_DTYPE_BF16)
+    gated_group_norm_kernel<bf16_t><<<grid, 256, lds, stream>>>(y, (const bf16_t*)x, ldx, (const bf16_t*)z, ldz, D, w, eps, (bf16_t*)out, H, dv, groups);
+  else
+    PICO_REQUIRE(false, "pico_gated_group_norm: unknown dtype %d", dtype);
+  PICO_LAUNCH_CHECK();
+  return 0;
+}

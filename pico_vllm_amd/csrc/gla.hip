@@ -350,7 +350,7 @@ extern "C" int pico_gla_scan(const void* x, int ldx, int dtype, int q_col, int k
 template <typename T>
 __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, const T* __restrict__ g, int ldg,
                                                      const float* __restrict__ w, float eps, T* __restrict__ out, int H,
-                                                     int dv) {
+                                                     int dv, int sigmoid_gate) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + ((size_t)t * H + h) * dv;
   float ss = 0.f;
@@ -361,19 +361,20 @@ __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o
   T* dst = out + ((size_t)t * H + h) * dv;
   for (int v = lane; v < dv; v += 64) {
     const float gv = load_f32(grow + v);
-    store_f32(dst + v, orow[v] * r * w[v] * (gv / (1.0f + expf(-gv))));
+    // the gate: silu(g), or sigmoid(g)
+    store_f32(dst + v, orow[v] * r * w[v] * ((sigmoid_gate ? 1.0f : gv) / (1.0f + expf(-gv))));
   }
 }
 
 extern "C" int pico_gla_out(const float* o, const void* g, int ldg, int dtype, const float* w, float eps, void* out, int T,
-                            int H, int dv, hipStream_t stream) {
+                            int H, int dv, int sigmoid_gate, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= H * dv && H <= 65535, "pico_gla_out: bad sizes");
   if (T == 0) return 0;
   const dim3 grid(T, H);
   if (dtype == PICO_DTYPE_F32)
-    gla_out_kernel<float><<<grid, 64, 0, stream>>>(o, (const float*)g, ldg, w, eps, (float*)out, H, dv);
+    gla_out_kernel<float><<<grid, 64, 0, stream>>>(o, (const float*)g, ldg, w, eps, (float*)out, H, dv, sigmoid_gate);
   else if (dtype == PICO_DTYPE_BF16)
-    gla_out_kernel<bf16_t><<<grid, 64, 0, stream>>>(o, (const bf16_t*)g, ldg, w, eps, (bf16_t*)out, H, dv);
+    gla_out_kernel<bf16_t><<<grid, 64, 0, stream>>>(o, (const bf16_t*)g, ldg, w, eps, (bf16_t*)out, H, dv, sigmoid_gate);
   else
     PICO_REQUIRE(false, "pico_gla_out: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

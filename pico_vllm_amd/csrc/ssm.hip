@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
   const int b = token_seq[t], first = cu_seqlens[b];
   const int slot = min(max(state_slots[b], 0), num_slots - 1);
   const float* hist = state + ((size_t)slot * C + c) * (N + taps - 1) + N;
-  float acc = bias[c];
+  float acc = bias ? bias[c] : 0.f;
   for (int j = 0; j < taps; j++) {
     const int src = t - (taps - 1) + j;                 // token index of this tap's input
     const float v = src >= first ? load_f32(x + (size_t)src * ldx + c) : hist[(taps - 1) + (src - first)];
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void causal_conv8_kernel(const bf16_t* __restr
   const int slot = min(max(state_slots[b], 0), num_slots - 1);
   float acc[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) acc[i] = bias[c0 + i];
+  for (int i = 0; i < 8; i++) acc[i] = bias ? bias[c0 + i] : 0.f;
   for (int j = 0; j < taps; j++) {
     const int src = t - (taps - 1) + j;
     float v[8];
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void causal_conv_step_kernel(const T* __restri
   if (cu_seqlens[b + 1] != t + 1 || slot < 0 || slot >= num_slots) return;
   float* hist = state + ((size_t)slot * C + c) * (N + taps - 1) + N;
   const float xv = load_f32(x + (size_t)t * ldx + c);
-  float acc = bias[c];
+  float acc = bias ? bias[c] : 0.f;
   float keep[SSM_MAX_TAPS];
   for (int j = 0; j < taps - 1; j++) {
     keep[j] = hist[j];
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void causal_conv_step_kernel(const T* __restri
 extern "C" int pico_causal_conv(const void* x, int ldx, int dtype, const float* w, const float* bias, const int* token_seq,
                                 const int* cu_seqlens, const int* state_slots, float* state, int num_slots, int T, int B,
                                 int C, int N, int taps, void* out, int single, hipStream_t stream) {
-  PICO_REQUIRE(T >= 0 && B >= 0 && C > 0 && N > 0 && taps >= 1 && taps <= SSM_MAX_TAPS && ldx >= C && num_slots > 0,
+  PICO_REQUIRE(T >= 0 && B >= 0 && C > 0 && N >= 0 && taps >= 1 && taps <= SSM_MAX_TAPS && ldx >= C && num_slots > 0,
                "pico_causal_conv: bad sizes (1 to %d taps)", SSM_MAX_TAPS);
   if (T == 0 || B == 0) return 0;
   const int cb = (C + 255) / 256;

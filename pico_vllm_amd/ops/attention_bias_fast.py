@@ -24,10 +24,14 @@ def supported(key_dim: int, value_dim: int) -> bool:
 class FastBiasAttention:
     def __init__(self, nq: int, nkv: int, key_dim: int, value_dim: int, scale: float, window: int = 0,
                  temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0, softcap: float = 0.0,
-                 keep_first: int = 0, gated: bool = False):
+                 keep_first: int = 0, gated: bool = False, chunk: int = 0, sink: bool = False, gate_heads: bool = False,
+                 v_div: int = 1, out_f32: bool = False):
         self.nq, self.nkv, self.dk, self.dv = nq, nkv, key_dim, value_dim
         self.scale, self.window, self.temp_coef, self.temp_every, self.slope_span = scale, window, temp_coef, temp_every, slope_span
         self.softcap, self.keep_first, self.gated = float(softcap), int(keep_first), bool(gated)
+        # chunked visibility instead of a window, a sink in the softmax, a gate of one number a head, several kv heads
+        # over one head of values, float32 output (see csrc/attention_bias.hip)
+        self.chunk, self.sink, self.gate_heads, self.v_div, self.out_f32 = int(chunk), bool(sink), bool(gate_heads), int(v_div), bool(out_f32)
         self.lib = library.attention_bias_library(key_dim, value_dim)
         if self.lib.pico_attnb_key_dim() != key_dim or self.lib.pico_attnb_value_dim() != value_dim:
             raise KernelError("attention library was built for other sizes")
@@ -37,7 +41,8 @@ class FastBiasAttention:
         self.tuned = None
         # (that kernel knows no cap on the scores, no kept first positions and no gate)
         if key_dim == value_dim and key_dim % 32 == 0 and attention_fast.supported(nq, nkv, key_dim, window) \
-                and not (self.softcap > 0 or (self.keep_first > 0 and window > 0) or self.gated):
+                and not (self.softcap > 0 or (self.keep_first > 0 and window > 0) or self.gated or self.chunk or self.sink
+                         or self.v_div != 1 or self.out_f32):
             self.tuned = attention_fast.FastAttention(nq, nkv, key_dim, window)
 
     def split(self, num_tokens: int) -> bool:
@@ -82,7 +87,7 @@ class FastBiasAttention:
         """q [T, >= nq * dk] bfloat16 (row stride free); any mixture of portions and single tokens; returns [T, nq * dv].
         ``gate`` [T, >= nq * dv] bfloat16 (8-byte aligned rows): the output is multiplied with sigmoid(gate)."""
         T = q.shape[0]
-        pages, P = _check_cache2(k_cache, v_cache, self.nkv, self.dk, self.dv)
+        pages, P = _check_cache2(k_cache, v_cache, self.nkv, self.dk, self.dv, self.nkv // self.v_div)
         if not q.is_cuda or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
             raise KernelError("matrix-core attention wants bfloat16 tensors on the GPU")
         if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < self.nq * self.dk or (T > 1 and q.stride(0) % 8) or q.data_ptr() % 16:
@@ -96,11 +101,11 @@ class FastBiasAttention:
         if P < 8 or P & (P - 1):
             raise KernelError("matrix-core attention wants pages of a power of two of at least 8 tokens")
         if gate is not None and (not gate.is_cuda or gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape[0] != T
-                                 or gate.stride(1) != 1 or gate.shape[1] < self.nq * self.dv or (T > 1 and gate.stride(0) % 4)
-                                 or gate.data_ptr() % 8):
+                                 or gate.stride(1) != 1 or gate.shape[1] < (self.nq if self.gate_heads else self.nq * self.dv)
+                                 or (not self.gate_heads and ((T > 1 and gate.stride(0) % 4) or gate.data_ptr() % 8))):
             raise KernelError("the gate must be bfloat16 [T, >= nq*dv] with unit stride along the row and 8-byte aligned rows")
         if out is None:
-            out = torch.empty(T, self.nq * self.dv, dtype=torch.bfloat16, device=q.device)
+            out = torch.empty(T, self.nq * self.dv, dtype=torch.float32 if self.out_f32 else torch.bfloat16, device=q.device)
         if split is None:
             split = self.split(T)
         if chunks is None:
@@ -116,7 +121,8 @@ class FastBiasAttention:
             _ptr(cu_seqlens), _ptr(positions), num_seqs, T, _ptr(out), self.nq, self.nkv, self.dk, self.dv, P, pages,
             c_float(self.scale), self.window, c_float(self.temp_coef), self.temp_every, c_float(self.slope_span),
             1 if split else 0, chunks, _ptr(parts_o), _ptr(parts_ml), c_float(self.softcap), self.keep_first, _ptr(gate),
-            0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), _stream()))
+            0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), self.chunk, 1 if self.sink else 0,
+            1 if self.gate_heads else 0, self.v_div, 1 if self.out_f32 else 0, _stream()))
         return out
 
     def __call__(self, qkv, cache, block_table, ctx, gate=None):
@@ -142,4 +148,6 @@ def choose(mixer) -> Optional[FastBiasAttention]:
         return None
     return FastBiasAttention(mixer.nq, mixer.nkv, mixer.dk, mixer.dv, mixer.scale, mixer.window, mixer.temp_coef,
                              mixer.temp_every, mixer.slope_span, getattr(mixer, "softcap", 0.0),
-                             getattr(mixer, "keep_first", 0), getattr(mixer, "gated", False))
+                             getattr(mixer, "keep_first", 0), getattr(mixer, "gated", False), getattr(mixer, "chunk", 0),
+                             getattr(mixer, "sink", False), getattr(mixer, "gate_heads", False), getattr(mixer, "v_div", 1),
+                             getattr(mixer, "out_f32", False))

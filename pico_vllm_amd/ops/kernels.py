@@ -595,14 +595,15 @@ def relu2(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     return out
 
 
-def _check_cache2(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, dk: int, dv: int):
-    """K pages [pages, nkv, P, dk]; V pages [pages, nkv, dv, P]."""
+def _check_cache2(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, dk: int, dv: int, nv: Optional[int] = None):
+    """K pages [pages, nkv, P, dk]; V pages [pages, nv, dv, P] (nv: nkv unless given)."""
+    nv = nkv if nv is None else nv
     if k_cache.dim() != 4 or v_cache.dim() != 4 or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("cache tensors must be contiguous and 4-dimensional")
     pages, h, P, dd = k_cache.shape
-    if (h, dd) != (nkv, dk) or tuple(v_cache.shape) != (pages, nkv, dv, P) or v_cache.dtype != k_cache.dtype:
+    if (h, dd) != (nkv, dk) or tuple(v_cache.shape) != (pages, nv, dv, P) or v_cache.dtype != k_cache.dtype:
         raise KernelError(f"cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
-                          f"{nkv} kv heads with keys of {dk} and values of {dv}")
+                          f"{nkv} kv heads with keys of {dk} and {nv} with values of {dv}")
     return pages, P
 
 
@@ -634,35 +635,43 @@ def attn_bias_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     positions: torch.Tensor, token_seq: torch.Tensor, nq: int, nkv: int, dk: int, dv: int, scale: float,
                     window: int = 0, temp_coef: float = 0.0, temp_every: int = 0, slope_span: float = 0.0,
                     out: Optional[torch.Tensor] = None, softcap: float = 0.0, keep_first: int = 0,
-                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    gate: Optional[torch.Tensor] = None, chunk: int = 0, sink: bool = False, gate_heads: bool = False,
+                    v_div: int = 1, out_f32: bool = False) -> torch.Tensor:
     """Attention with a distance penalty slope_h (i - j), slope_h = 2^(-slope_span (h + 1) / nq), and the query
     temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on the scores.  q: [T, >= nq * dk]; returns [T, nq * dv].
     ``softcap`` > 0: scores <- softcap tanh(scores / softcap).  ``keep_first``: with a window, keys at positions below it
-    stay visible.  ``gate`` [T, >= nq * dv] (row stride free): the output is multiplied with sigmoid(gate)."""
+    stay visible.  ``gate`` [T, >= nq * dv] (row stride free): the output is multiplied with sigmoid(gate); with
+    ``gate_heads`` the gate is [T, >= nq], one number a head.  ``chunk`` > 0 (instead of a window): key j <= i is seen iff
+    floor(i / chunk) == floor(j / chunk).  ``sink``: the softmax's denominator gains a 1.  ``v_div``: kv head g reads value
+    head g // v_div (the value pages hold nkv // v_div heads).  ``out_f32``: the output is float32 whatever q's dtype."""
     _gpu(q, k_cache, v_cache, block_table, positions, token_seq, gate)
     T = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nq * dk:
         raise KernelError("q must be [T, >= nq*dk] with unit stride along the row")
-    pages, P = _check_cache2(k_cache, v_cache, nkv, dk, dv)
+    if v_div < 1 or nkv % v_div or chunk < 0 or (chunk and window):
+        raise KernelError("attention: kv heads share values in whole groups; chunks or a window, not both")
+    pages, P = _check_cache2(k_cache, v_cache, nkv, dk, dv, nkv // v_div)
     if k_cache.dtype != q.dtype:
         raise KernelError("cache and activations differ in dtype")
     _i32(positions, "positions", T)
     _i32(token_seq, "token_seq", T)
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
         raise KernelError("block_table must be contiguous int32 [sequences, pages]")
+    odt = torch.float32 if out_f32 else q.dtype
     if out is None:
-        out = torch.empty(T, nq * dv, dtype=q.dtype, device=q.device)
-    elif out.shape != (T, nq * dv) or out.dtype != q.dtype or not out.is_contiguous():
+        out = torch.empty(T, nq * dv, dtype=odt, device=q.device)
+    elif out.shape != (T, nq * dv) or out.dtype != odt or not out.is_contiguous():
         raise KernelError("attention: out has the wrong shape or dtype")
     if gate is not None and (gate.dtype != q.dtype or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != T
-                             or gate.shape[1] < nq * dv):
-        raise KernelError(f"attention: the gate must be [T, >= {nq * dv}] of the activations' dtype")
+                             or gate.shape[1] < (nq if gate_heads else nq * dv)):
+        raise KernelError(f"attention: the gate must be [T, >= {nq if gate_heads else nq * dv}] of the activations' dtype")
     lib = library.core()
     _check(lib, lib.pico_attn_bias_plain(_ptr(q), q.stride(0) if T > 1 else q.shape[1], _dt(q), _ptr(k_cache), _ptr(v_cache),
                                          _ptr(block_table), block_table.shape[1], _ptr(positions), _ptr(token_seq), _ptr(out),
                                          T, nq, nkv, dk, dv, P, window, c_float(scale), c_float(temp_coef), temp_every,
                                          c_float(slope_span), pages, c_float(softcap), keep_first, _ptr(gate),
-                                         0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), _stream()))
+                                         0 if gate is None else (gate.stride(0) if T > 1 else gate.shape[1]), chunk,
+                                         1 if sink else 0, 1 if gate_heads else 0, v_div, 1 if out_f32 else 0, _stream()))
     return out
 
 
@@ -766,9 +775,10 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, log_decay: Opt
     return out
 
 
-def gla_out(o: torch.Tensor, x: torch.Tensor, g_col: int, weight: torch.Tensor, eps: float, heads: int, dv: int) -> torch.Tensor:
+def gla_out(o: torch.Tensor, x: torch.Tensor, g_col: int, weight: torch.Tensor, eps: float, heads: int, dv: int,
+            sigmoid_gate: bool = False) -> torch.Tensor:
     """[T, heads * dv] of x's dtype: every head of ``o`` (float32) RMS-normed over its dv entries with ``weight`` [dv],
-    times silu of the gate (columns g_col .. of x)."""
+    times silu of the gate (columns g_col .. of x), or with ``sigmoid_gate`` times its sigmoid."""
     _gpu(o, x, weight)
     T = o.shape[0]
     if o.dtype != torch.float32 or tuple(o.shape) != (T, heads * dv) or not o.is_contiguous():
@@ -780,7 +790,7 @@ def gla_out(o: torch.Tensor, x: torch.Tensor, g_col: int, weight: torch.Tensor, 
     out = torch.empty(T, heads * dv, dtype=x.dtype, device=x.device)
     lib = library.core()
     _check(lib, lib.pico_gla_out(_ptr(o), _ptr(x[:, g_col:]), x.stride(0) if T > 1 else x.shape[1], _dt(x), _ptr(weight),
-                                 c_float(eps), _ptr(out), T, heads, dv, _stream()))
+                                 c_float(eps), _ptr(out), T, heads, dv, 1 if sigmoid_gate else 0, _stream()))
     return out
 
 
@@ -1122,7 +1132,7 @@ def causal_conv(x: torch.Tensor, channels: int, w: torch.Tensor, bias: torch.Ten
         raise KernelError("causal_conv: the rows do not hold the channels")
     if w.dtype != torch.float32 or tuple(w.shape) != (taps, channels) or not w.is_contiguous() or not 1 <= taps <= SSM_MAX_TAPS:
         raise KernelError(f"causal_conv: the taps are contiguous float32 [1 to {SSM_MAX_TAPS}, {channels}]")
-    _vec(bias, channels, "the convolution's bias")
+    _vec(bias, channels, "the convolution's bias")          # None: no bias
     if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (channels, n_state + taps - 1) or not state.is_contiguous():
         raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {channels}, {n_state + taps - 1}]")
     B = ctx.num_seqs
@@ -1197,3 +1207,239 @@ def moe_router_top_softmax(x: torch.Tensor, w_router: torch.Tensor, bias: Option
     _check(lib, lib.pico_moe_router_top_softmax(_ptr(x), x.stride(0) if T > 1 else D, _dt(x), _ptr(w_router), _ptr(bias), T,
                                                 experts, rows - experts, D, top, _ptr(z), _ptr(chosen), _ptr(weights), _stream()))
     return chosen, weights, z
+
+
+# ---- norms on what a sublayer returns; the stream's own norm ---------------------------------------------------------------
+def _delta_like(resid, y, who):
+    T, H = resid.shape
+    if y.dim() == 3:
+        if y.dtype != torch.float32:
+            raise KernelError(f"{who}: a stack of partial sums must be float32")
+    elif y.dim() != 2:
+        raise KernelError(f"{who}: an output is [T, H] or a stack [S, T, H]")
+    if tuple(y.shape[-2:]) != (T, H) or not y.is_contiguous():
+        raise KernelError(f"{who}: an output must be contiguous and shaped like the residual stream")
+    return y.shape[0] if y.dim() == 3 else 1
+
+
+def norm_add(resid: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, copy_dtype: Optional[torch.dtype] = None,
+             y2: Optional[torch.Tensor] = None, weight1: Optional[torch.Tensor] = None,
+             weight2: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """resid (float32 [T, H], in place) += rms(y) * weight.  With ``y2``: y and y2 are each RMS-normed with their own
+    weights (weight1, weight2), half their sum takes y's place.  y, y2: [T, H], or float32 stacks [S, T, H] whose slabs are
+    added up first.  ``copy_dtype``: also returns the new rows in that dtype (what the next sublayer reads)."""
+    _gpu(resid, y, weight, y2, weight1, weight2)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    _vec(weight, H, "norm weight")
+    s1 = _delta_like(resid, y, "norm_add")
+    s2 = 1
+    if y2 is not None:
+        s2 = _delta_like(resid, y2, "norm_add")
+        if weight1 is None or weight2 is None:
+            raise KernelError("norm_add: two outputs come with a weight each")
+        _vec(weight1, H, "norm weight"); _vec(weight2, H, "norm weight")
+    copy = torch.empty(T, H, dtype=copy_dtype, device=resid.device) if copy_dtype is not None else None
+    lib = library.core()
+    _check(lib, lib.pico_norm_add(_ptr(resid), _ptr(y), _dt(y), s1, _ptr(weight1), _ptr(y2), _dt(y2) if y2 is not None else F32, s2,
+                                  _ptr(weight2), c_ll(T * H), _ptr(weight), c_float(eps), _ptr(copy),
+                                  _DT[copy_dtype] if copy_dtype is not None else F32, T, H, _stream()))
+    return copy
+
+
+def stream_rmsnorm(resid: torch.Tensor, weight: torch.Tensor, eps: float, copy_dtype: Optional[torch.dtype] = None):
+    """resid (float32 [T, H]) <- rms(resid) * weight in place; ``copy_dtype``: also returns the rows in that dtype."""
+    _gpu(resid, weight)
+    T, H = resid.shape
+    if resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise KernelError("the residual stream must be contiguous float32")
+    _vec(weight, H, "norm weight")
+    copy = torch.empty(T, H, dtype=copy_dtype, device=resid.device) if copy_dtype is not None else None
+    lib = library.core()
+    _check(lib, lib.pico_stream_rmsnorm(_ptr(resid), _ptr(weight), c_float(eps), _ptr(copy),
+                                        _DT[copy_dtype] if copy_dtype is not None else F32, T, H, _stream()))
+    return copy
+
+
+def cast_rows(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """A contiguous float32 tensor in the activations' dtype (float32: itself)."""
+    _gpu(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("cast_rows: a contiguous float32 tensor")
+    if dtype == torch.float32:
+        return x
+    out = torch.empty_like(x, dtype=dtype)
+    lib = library.core()
+    _check(lib, lib.pico_cast_rows(_ptr(x), _ptr(out), _DT[dtype], c_ll(x.numel()), _stream()))
+    return out
+
+
+# ---- what stands between the q/k/v product and an attention that norms its queries and keys --------------------------------
+QK_NORM_NONE, QK_NORM_UNIT, QK_NORM_ROW = 0, 1, 2
+
+
+def qk_norm_store(x: torch.Tensor, q_col: int, k_col: int, v_col: int, nq: int, nk: int, nv: int, dk: int, dv: int, maps: int,
+                  norm_mode: int, wq: Optional[torch.Tensor], wk: Optional[torch.Tensor], eps: float,
+                  cos_sin: Optional[torch.Tensor], rotary_dim: int, slots: Optional[torch.Tensor],
+                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+    """RMS norm of the nq query and nk key units of dk entries in every row of x (QK_NORM_UNIT: every unit by itself,
+    weights [dk]; QK_NORM_ROW: all units of a row at once, weights [nq * dk] and [nk * dk]), then the first ``rotary_dim``
+    entries of every unit turned (entry i with i + rotary_dim / 2; ``cos_sin`` from ``rope_table``).  Returns the queries
+    [T, nq * dk]; with ``maps`` > 1 (a head holds that many units) in the order (kv group, map, head in group).  Keys go
+    to ``k_cache`` [pages, nk, P, dk] and columns v_col .. of x, as they are, to ``v_cache`` [pages, nv, dv, P] at
+    ``slots`` (negative: nothing); without a cache only the queries are made."""
+    _gpu(x, wq, wk, cos_sin, slots, k_cache, v_cache)
+    T = x.shape[0]
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("qk_norm_store: x must be [T, columns] with unit stride along the row")
+    if maps < 1 or nq % maps or nk % maps or (nq // maps) % (nk // maps):
+        raise KernelError("qk_norm_store: query heads are a multiple of kv heads, and both hold whole maps")
+    if x.shape[1] < max(q_col + nq * dk, k_col + nk * dk, v_col + nv * dv):
+        raise KernelError("qk_norm_store: the rows do not hold q, k and v")
+    if norm_mode != QK_NORM_NONE:
+        n = dk if norm_mode == QK_NORM_UNIT else None
+        _vec(wq, n or nq * dk, "the queries' norm weight"); _vec(wk, n or nk * dk, "the keys' norm weight")
+        if wq is None or wk is None:
+            raise KernelError("qk_norm_store: a norm needs its weights")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= dk:
+        raise KernelError(f"qk_norm_store: {rotary_dim} turned entries do not fit a unit of {dk}")
+    _check_table(cos_sin, T, rotary_dim // 2)
+    pages = P = 0
+    if k_cache is not None:
+        pages, P = _check_cache2(k_cache, v_cache, nk, dk, dv, nv)
+        if k_cache.dtype != x.dtype:
+            raise KernelError("cache and activations differ in dtype")
+        _i32(slots, "slots", T)
+    q_out = torch.empty(T, nq * dk, dtype=x.dtype, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_qk_norm_store(_ptr(x), _dt(x), x.stride(0) if T > 1 else x.shape[1], q_col, k_col, v_col, nq, nk, nv, dk,
+                                       dv, maps, norm_mode, _ptr(wq), _ptr(wk), c_float(eps),
+                                       _ptr(cos_sin) if rotary_dim else None, rotary_dim, _ptr(slots), _ptr(q_out), _ptr(k_cache),
+                                       _ptr(v_cache), T, P, pages, _stream()))
+    return q_out
+
+
+def diff_combine(a: torch.Tensor, lam: float, eps: float, mult: float, heads: int, kv_heads: int, dv: int,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """Two attention maps a head into one output: a float32 [T, 2 * heads * dv] in the order (kv group, map, head in group);
+    o = a1 - lam * a2, over its root mean square (eps inside), times ``mult``.  Returns [T, heads * dv] in head order."""
+    _gpu(a)
+    T = a.shape[0]
+    if a.dtype != torch.float32 or tuple(a.shape) != (T, 2 * heads * dv) or not a.is_contiguous() or heads % kv_heads:
+        raise KernelError(f"diff_combine: the maps' outputs must be contiguous float32 [T, {2 * heads * dv}]")
+    out = torch.empty(T, heads * dv, dtype=out_dtype, device=a.device)
+    lib = library.core()
+    _check(lib, lib.pico_diff_combine(_ptr(a), c_float(lam), c_float(eps), c_float(mult), _ptr(out), _DT[out_dtype], T, heads,
+                                      kv_heads, dv, _stream()))
+    return out
+
+
+# ---- recurrent mixers with a matrix state: the delta rule, state-space duality ---------------------------------------------
+DELTA_MAX_KEY_DIM = 512
+
+
+def delta_prep(x: torch.Tensor, q_col: int, k_col: int, y: torch.Tensor, b_col: int, a_col: int, a2: torch.Tensor,
+               dt_bias: torch.Tensor, a_log: torch.Tensor, qscale: float, heads: int, kv_heads: int, dk: int):
+    """What enters the delta rule's walk, in float32: unit vectors q (times qscale) and k per q/k head [T, kv_heads * dk]
+    from columns q_col .., k_col .. of x; decays g = exp(-exp(a_log_h) softplus(a2 (y[:, a_col : a_col + R]) + dt_bias))
+    [T, heads * dk]; beta = sigmoid(y[:, b_col : b_col + heads]) [T, heads]."""
+    _gpu(x, y, a2, dt_bias, a_log)
+    T = x.shape[0]
+    C, R = a2.shape
+    if x.dim() != 2 or y.dim() != 2 or x.stride(1) != 1 or y.stride(1) != 1 or y.shape[0] != T or x.dtype != y.dtype:
+        raise KernelError("delta_prep: x and y are [T, columns] of one dtype with unit stride along the row")
+    if C != heads * dk or a2.dtype != x.dtype or not a2.is_contiguous() or heads % kv_heads:
+        raise KernelError(f"delta_prep: a2 must be contiguous [{heads * dk}, R] of the activations' dtype")
+    if x.shape[1] < max(q_col, k_col) + kv_heads * dk or y.shape[1] < max(b_col + heads, a_col + R):
+        raise KernelError("delta_prep: the rows do not hold what is read")
+    _vec(dt_bias, heads * dk, "the decay's bias"); _vec(a_log, heads, "A_log")
+    dev = x.device
+    qn = torch.empty(T, kv_heads * dk, dtype=torch.float32, device=dev)
+    kn = torch.empty(T, kv_heads * dk, dtype=torch.float32, device=dev)
+    g = torch.empty(T, heads * dk, dtype=torch.float32, device=dev)
+    beta = torch.empty(T, heads, dtype=torch.float32, device=dev)
+    lib = library.core()
+    _check(lib, lib.pico_delta_prep(_ptr(x), x.stride(0) if T > 1 else x.shape[1], q_col, k_col, _ptr(y),
+                                    y.stride(0) if T > 1 else y.shape[1], b_col, a_col, _dt(x), _ptr(a2), _ptr(dt_bias), _ptr(a_log),
+                                    c_float(qscale), _ptr(qn), _ptr(kn), _ptr(g), _ptr(beta), T, heads, kv_heads, dk, R, _stream()))
+    return qn, kn, g, beta
+
+
+def ssd_prep(bc: torch.Tensor, b_col: int, c_col: int, n: int, y: torch.Tensor, dt_col: int, dt_bias: torch.Tensor,
+             a_log: torch.Tensor, heads: int):
+    """What enters a state-space walk, in float32: B and C (n columns each of bc from b_col, c_col) widened;
+    dt = softplus(y[:, dt_col : dt_col + heads] + dt_bias) and the decay exp(-exp(a_log) dt), both [T, heads]."""
+    _gpu(bc, y, dt_bias, a_log)
+    T = bc.shape[0]
+    if bc.dim() != 2 or y.dim() != 2 or bc.stride(1) != 1 or y.stride(1) != 1 or y.shape[0] != T or bc.dtype != y.dtype:
+        raise KernelError("ssd_prep: bc and y are [T, columns] of one dtype with unit stride along the row")
+    if bc.shape[1] < max(b_col, c_col) + n or y.shape[1] < dt_col + heads:
+        raise KernelError("ssd_prep: the rows do not hold what is read")
+    _vec(dt_bias, heads, "dt bias"); _vec(a_log, heads, "A_log")
+    dev = bc.device
+    bf = torch.empty(T, n, dtype=torch.float32, device=dev)
+    cf = torch.empty(T, n, dtype=torch.float32, device=dev)
+    g = torch.empty(T, heads, dtype=torch.float32, device=dev)
+    dt = torch.empty(T, heads, dtype=torch.float32, device=dev)
+    lib = library.core()
+    _check(lib, lib.pico_ssd_prep(_ptr(bc), bc.stride(0) if T > 1 else bc.shape[1], b_col, c_col, n, _ptr(y),
+                                  y.stride(0) if T > 1 else y.shape[1], dt_col, _dt(bc), _ptr(dt_bias), _ptr(a_log), _ptr(bf), _ptr(cf),
+                                  _ptr(g), _ptr(dt), T, heads, _stream()))
+    return bf, cf, g, dt
+
+
+def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, cu_seqlens: torch.Tensor,
+               state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, kv_heads: int, dk: int, dv: int,
+               delta: bool = True) -> torch.Tensor:
+    """The walk S <- diag(g_t) S; u = beta_t (v_t - S^T k_t) (``delta``; else u = beta_t v_t); S <- S + k_t u^T;
+    o_t = S^T q_t, for every sequence of the step from its state slot (``state`` float32 [slots, heads, dk, dv], updated in
+    place).  q, k float32 [T, kv_heads * dk] (head h reads q/k head h // (heads // kv_heads)); v [T, >= heads * dv] (row
+    stride free); g float32 [T, heads * dk] (a decay a key channel) or [T, heads] (one a head); beta float32 [T, heads].
+    Returns o float32 [T, heads * dv]."""
+    _gpu(q, k, v, g, beta, cu_seqlens, state_slots, state)
+    T = q.shape[0]
+    for t, name in ((q, "q"), (k, "k")):
+        if t.dtype != torch.float32 or tuple(t.shape) != (T, kv_heads * dk) or not t.is_contiguous():
+            raise KernelError(f"delta_scan: {name} must be contiguous float32 [T, {kv_heads * dk}]")
+    if v.dim() != 2 or v.shape[0] != T or v.stride(1) != 1 or v.shape[1] < heads * dv:
+        raise KernelError("delta_scan: the rows do not hold the values")
+    if g.dtype != torch.float32 or not g.is_contiguous() or tuple(g.shape) not in ((T, heads * dk), (T, heads)):
+        raise KernelError("delta_scan: the decays are contiguous float32, one a key channel or one a head")
+    g_channels = tuple(g.shape) == (T, heads * dk)
+    if beta.dtype != torch.float32 or tuple(beta.shape) != (T, heads) or not beta.is_contiguous():
+        raise KernelError(f"delta_scan: beta must be contiguous float32 [T, {heads}]")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dk, dv) or not state.is_contiguous():
+        raise KernelError(f"delta_scan: the state must be contiguous float32 [slots, {heads}, {dk}, {dv}]")
+    if dk > DELTA_MAX_KEY_DIM or heads % kv_heads:
+        raise KernelError(f"delta_scan: at most {DELTA_MAX_KEY_DIM} key channels a head; heads a multiple of q/k heads")
+    _i32(cu_seqlens, "cu_seqlens", num_seqs + 1)
+    _i32(state_slots, "state_slots", num_seqs)
+    out = torch.empty(T, heads * dv, dtype=torch.float32, device=q.device)
+    lib = library.core()
+    _check(lib, lib.pico_delta_scan(_ptr(q), _ptr(k), _ptr(v), v.stride(0) if T > 1 else v.shape[1], _dt(v), _ptr(g),
+                                    1 if g_channels else 0, _ptr(beta), _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out),
+                                    num_seqs, heads, kv_heads, dk, dv, state.shape[0], 1 if delta else 0, _stream()))
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, x: torch.Tensor, z: torch.Tensor, d: torch.Tensor, weight: torch.Tensor, eps: float,
+                     heads: int, dv: int, groups: int) -> torch.Tensor:
+    """((y + d_h x) * silu(z)) RMS-normed in ``groups`` equal parts of the row, times ``weight``; y float32 [T, heads * dv];
+    x, z [T, >= heads * dv] of the activations' dtype (row strides free); returns [T, heads * dv] of that dtype."""
+    _gpu(y, x, z, d, weight)
+    T, n = y.shape[0], heads * dv
+    if y.dtype != torch.float32 or tuple(y.shape) != (T, n) or not y.is_contiguous():
+        raise KernelError(f"gated_group_norm: y must be contiguous float32 [T, {n}]")
+    for t in (x, z):
+        if t.dim() != 2 or t.shape[0] != T or t.stride(1) != 1 or t.shape[1] < n or t.dtype != x.dtype:
+            raise KernelError("gated_group_norm: x and z are [T, >= heads * dv] of one dtype with unit stride along the row")
+    if groups < 1 or n % groups:
+        raise KernelError(f"gated_group_norm: {n} entries are not {groups} equal parts")
+    _vec(d, heads, "D"); _vec(weight, n, "norm weight")
+    out = torch.empty(T, n, dtype=x.dtype, device=x.device)
+    lib = library.core()
+    _check(lib, lib.pico_gated_group_norm(_ptr(y), _ptr(x), x.stride(0) if T > 1 else x.shape[1], _ptr(z),
+                                          z.stride(0) if T > 1 else z.shape[1], _dt(x), _ptr(d), _ptr(weight), c_float(eps), _ptr(out),
+                                          T, heads, dv, groups, _stream()))
+    return out

@@ -28,7 +28,8 @@ HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC",
              "-Wno-unused-command-line-argument"]
 
 CORE_SOURCES = ("errors.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "gemm_skinny.hip", "attention_ref.hip", "attention_bias.hip",
-                "moe.hip", "moe_mfma.hip", "sampling.hip", "rope_pairs.hip", "gla.hip", "layernorm.hip", "latent.hip", "ssm.hip")
+                "moe.hip", "moe_mfma.hip", "sampling.hip", "rope_pairs.hip", "gla.hip", "layernorm.hip", "latent.hip", "ssm.hip",
+                "postnorm.hip", "qk_prep.hip", "delta.hip")
 
 ATTN_SOURCES = ("errors.hip", "attention_mfma.hip")
 

@@ -171,3 +171,59 @@ class ScaledMixerOnlyBlock(ScaledPreNormBlock):
         h = p["norm1"].add_norm(resid, pending)
         kernels.scaled_add(resid, p["mixer"].forward(h, ctx, cache), scale=self.s1)
         return resid, None
+
+
+@register_part("block", "postnorm")
+class PostNormBlock(Block):
+    """x += norm1(mixer(x)); x += norm2(ff(x)): the sublayers read the residual stream itself, and the norm stands on
+    what a sublayer returns.  Each sum happens inside its norm's launch, in float32 (the next sublayer needs the new
+    stream, so nothing is handed on as pending), and the same launch leaves the stream's rows in the activations' dtype
+    for the next sublayer.  A mixer that offers ``forward_pair(h, ctx, cache) -> (a, wa, b, wb)`` (two mixers side by
+    side) has both outputs normed with their own weights and averaged inside that launch too."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ff": "feed_forward"}
+    graph_safe_prompts = True
+
+    def _rows(self, resid, ctx):
+        from .norm import stream_rows
+        return stream_rows(resid, ctx, self.parts["norm1"].act_dtype)
+
+    def _join(self, norm, resid, y, ctx, pair=None):
+        from .norm import STREAM_COPY
+        act = norm.act_dtype
+        want = None if act == resid.dtype else act
+        if pair is None:
+            copy = kernels.norm_add(resid, y, norm.weight, norm.eps, want)
+        else:
+            a, wa, b, wb = pair
+            copy = kernels.norm_add(resid, a, norm.weight, norm.eps, want, y2=b, weight1=wa, weight2=wb)
+        if copy is not None:
+            ctx.shared[STREAM_COPY] = (resid, copy)
+
+    def _mixer(self, resid, pending, ctx, cache):
+        p = self.parts
+        if pending is not None:                                   # a block in front that hands a delta on
+            for d in (pending if pending.dim() == 3 else (pending,)):
+                kernels.residual_add(resid, d)
+            ctx.shared.pop("stream_copy", None)
+        h = self._rows(resid, ctx)
+        pair = getattr(p["mixer"], "forward_pair", None)
+        if pair is not None:
+            self._join(p["norm1"], resid, None, ctx, pair=pair(h, ctx, cache))
+        else:
+            self._join(p["norm1"], resid, p["mixer"].forward(h, ctx, cache), ctx)
+
+    def forward(self, resid, pending, ctx, cache):
+        self._mixer(resid, pending, ctx, cache)
+        p = self.parts
+        self._join(p["norm2"], resid, p["ff"].forward(self._rows(resid, ctx), ctx), ctx)
+        return resid, None
+
+
+@register_part("block", "postnorm_mixer_only")
+class PostNormMixerOnlyBlock(PostNormBlock):
+    """x += norm1(mixer(x)) and nothing else: the arrangement above for a layer without a feed-forward."""
+    slot_categories = {"norm1": "norm", "mixer": "mixer"}
+
+    def forward(self, resid, pending, ctx, cache):
+        self._mixer(resid, pending, ctx, cache)
+        return resid, None

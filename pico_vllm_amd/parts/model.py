@@ -9,7 +9,7 @@ from ..config.registry import load_model_description
 from ..ops import kernels
 from ..ops.linear import Linear
 from ..weights.loader import load_checkpoint
-from . import attention, attention_bias, attention_gated, block, gla, latent_attention, mlp, moe, norm, positions, retention, rotary, ssm  # noqa: F401  (register the parts)
+from . import attention, attention_bias, attention_chunked, attention_diff, attention_gated, block, delta, gla, latent_attention, mlp, moe, norm, pair, positions, retention, rotary, ssm  # noqa: F401  (register the parts)
 from .base import Block, StepContext
 from .registry import build_part, part_class
 from .spec import CacheSpec, ModelSpec, ParamSpec
@@ -100,9 +100,18 @@ class DecoderModel:
                     raise ValueError(f"run entry {i} cannot use the cache of entry {e.cache_of}: different cache needs")
 
     def cache_specs(self) -> Dict[int, CacheSpec]:
-        """CacheSpec by cache id: the index of the run entry that owns the cache; -(k + 1) for the k-th part around the
-        layers (``before_layers``, then ``after_layers``) that keeps a state."""
-        out = {i: self.layers[self.spec.run_order[i].layer].mixer.cache_spec() for i in self.spec.cache_owners()}
+        """CacheSpec by cache id: the index of the run entry that owns the cache (a tuple that starts with it for the
+        parts of a mixer that keeps several caches); -(k + 1) for the k-th part around the layers (``before_layers``,
+        then ``after_layers``) that keeps a state."""
+        out = {}
+        for i in self.spec.cache_owners():
+            cs = self.layers[self.spec.run_order[i].layer].mixer.cache_spec()
+            if cs.kind == "several":
+                # every part is a cache of its own, under the id (run entry, indices that lead to the part)
+                for path, leaf in cs.leaves():
+                    out[(i,) + path] = leaf
+            else:
+                out[i] = cs
         for k, (_, part) in enumerate(self.before + self.after):
             cs = part.cache_spec()
             if cs.kind == "state":
@@ -183,6 +192,7 @@ class DecoderModel:
         for i, e in enumerate(self.spec.run_order):
             if e.add_input:
                 kernels.residual_add(resid, entered)       # what is pending joins later; the sums are float32
+                ctx.shared.pop("stream_copy", None)            # a copy of the stream in the activations' dtype is stale now
             # a run that names another run's cache reads it and stores nothing of its own
             resid, pending = self.layers[e.layer].forward(resid, pending, ctx,
                                                           storage.layer(self.spec.cache_id(i), read_only=e.cache_of is not None))

@@ -6,7 +6,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..ops import kernels
-from .base import DeferredNorm, Norm
+from .base import DeferredNorm, Norm, StreamPart
 from .registry import register_part
 from .spec import ParamSpec
 
@@ -69,3 +69,42 @@ class LayerNorm(Norm):
         if delta is not None and delta.dim() == 3 and delta.shape[0] > kernels.LN_MAX_SLABS:
             raise ValueError(f"a layer norm's launch adds at most {kernels.LN_MAX_SLABS} partial sums")
         return kernels.add_layernorm(resid, delta, self.weight, self.bias, self.eps, self.act_dtype, rows, delta_scale)
+
+
+# what a step's parts share: the residual stream's rows in the activations' dtype, made by whoever wrote the stream last
+# (a sublayer that reads the stream itself, not a norm of it, takes them from here): (the stream tensor, its copy)
+STREAM_COPY = "stream_copy"
+
+
+def stream_rows(resid: torch.Tensor, ctx, act_dtype: torch.dtype) -> torch.Tensor:
+    """The residual stream in the activations' dtype: the stream itself in the 32-bit engine, else the copy that the
+    kernel which last wrote the stream left, or a fresh one."""
+    if act_dtype == torch.float32:
+        return resid
+    have = ctx.shared.get(STREAM_COPY)
+    if have is not None and have[0] is resid:
+        return have[1]
+    return kernels.cast_rows(resid, act_dtype)
+
+
+@register_part("stream", "stream_rms_norm")
+class StreamRMSNorm(StreamPart):
+    """x <- x / sqrt(mean(x^2) + eps) * weight on the residual stream itself, in float32 (a norm of the embeddings in
+    front of the first layer).  Leaves the rows in the activations' dtype for the first sublayer that reads the stream."""
+    graph_safe_prompts = True
+
+    def __init__(self, size: int, eps: float, act_dtype: torch.dtype = torch.bfloat16, weight_name: str = "weight"):
+        self.size, self.eps, self.act_dtype, self.weight_name = size, eps, act_dtype, weight_name
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        return [ParamSpec(self.weight_name, (self.size,), role="norm")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], device, dtype) -> None:
+        self.weight = tensors[self.weight_name].to(device=device, dtype=torch.float32).contiguous()
+
+    def forward(self, resid, ctx):
+        copy = kernels.stream_rmsnorm(resid, self.weight, self.eps, None if self.act_dtype == torch.float32 else self.act_dtype)
+        if copy is not None:
+            ctx.shared[STREAM_COPY] = (resid, copy)
+        return resid

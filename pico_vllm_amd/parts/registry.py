@@ -26,7 +26,7 @@ def register_part(category: str, kind: str, cls=None):
 def _register_own_parts() -> None:
     """The parts of this package register themselves when their modules load; whoever asks the registry first
     makes sure they have."""
-    from . import attention, attention_bias, attention_gated, block, gla, latent_attention, mlp, moe, norm, positions, retention, rotary, ssm  # noqa: F401
+    from . import attention, attention_bias, attention_chunked, attention_diff, attention_gated, block, delta, gla, latent_attention, mlp, moe, norm, pair, positions, retention, rotary, ssm  # noqa: F401
 
 
 def part_class(category: str, kind: str):

@@ -64,19 +64,38 @@ class CacheSpec:
     and their layout inside a page; the cache only allocates them, one allocation a tensor and
     layer, and hands them to the mixer by name); ``window`` > 0 means only the last ``window``
     positions are ever read again, so older pages can be given back early; except that the first ``keep_first``
-    positions of a request stay readable whatever the window (their pages are never given back early).
+    positions of a request stay readable whatever the window (their pages are never given back early);
+    ``chunk`` > 0 (instead of a window) means a position reads only positions of its own chunk of that many, counted
+    from position 0, so the pages of earlier chunks can be given back.
     kind "state": a fixed-size tensor of ``state_shape`` per request.
     kind "none": nothing.
+    kind "several": what ``parts`` lists, each a cache of its own (a mixer made of two mixers side by side; a recurrent
+    state and a convolution's last inputs).  The mixer is handed a list of cache entries in the order of ``parts``
+    (nested where a part is itself "several").
     Layers with equal specs share a pool of page ids and a block table per request.
     """
     kind: str = "none"
     window: int = 0
     keep_first: int = 0
+    chunk: int = 0
     page_tensors: Tuple[PageTensor, ...] = ()
     state_shape: Tuple[int, ...] = ()
     state_dtype: str = "float32"
+    parts: Tuple["CacheSpec", ...] = ()
+
+    def leaves(self, path: Tuple[int, ...] = ()):
+        """(path, spec) of every cache this spec asks for: itself under the empty path, or the parts of a "several"
+        under the indices that lead to them."""
+        if self.kind != "several":
+            return [(path, self)]
+        out = []
+        for k, p in enumerate(self.parts):
+            out += p.leaves(path + (k,))
+        return out
 
     def __post_init__(self):
+        if self.kind == "several" and not self.parts:
+            raise ValueError("a cache of several parts lists them")
         if self.kind == "paged_kv":
             names = [t.name for t in self.page_tensors]
             if not names or len(set(names)) != len(names):
