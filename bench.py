@@ -58,10 +58,13 @@ SHAPES = {"1.5b": ("Qwen2.5-1.5B shape", preset("1.5b")), "7b": ("Qwen2.5-7B sha
           "nasedra-1.5b": ("Nasedra at the 1.5B shape's sizes", preset("nasedra-1.5b")),
           "nasedra-7b": ("Nasedra at the 7B shape's sizes", preset("nasedra-7b")),
           "dikolix-1.5b": ("Dikolix at the 1.5B shape's sizes", preset("dikolix-1.5b")),
-          "dikolix-7b": ("Dikolix at the 7B shape's sizes", preset("dikolix-7b"))}
+          "dikolix-7b": ("Dikolix at the 7B shape's sizes", preset("dikolix-7b")),
+          "vagelix-1.5b": ("Vagelix at the 1.5B shape's sizes", preset("vagelix-1.5b")),
+          "vagelix-7b": ("Vagelix at the 7B shape's sizes", preset("vagelix-7b"))}
 # --workload designs: (a design's configuration, the closest existing model at equal size)
 DESIGN_PAIRS = (("lerazen-1.5b", "1.5b"), ("lerazen-7b", "7b"), ("nasedra-1.5b", "1.5b"), ("nasedra-7b", "7b"),
-                ("dikolix-1.5b", "nasedra-1.5b"), ("dikolix-7b", "nasedra-7b"))
+                ("dikolix-1.5b", "nasedra-1.5b"), ("dikolix-7b", "nasedra-7b"),
+                ("vagelix-1.5b", "nasedra-1.5b"), ("vagelix-7b", "nasedra-7b"))
 CONFIG = SHAPES["1.5b"][1]   # the shape being measured (set in main)
 CONTEXT = 4096
 PREFILL_TOKENS = 2048

@@ -106,6 +106,29 @@ DESIGN_PRESETS.update({
 })
 
 
+def _vagelix(vocab, width, layers, heads, kv_heads, dim, ff, chunk=1024, delta_dim=64, ssd_dim=64, ssd_state=128,
+             ssd_groups=2) -> Dict:
+    """A Vagelix configuration of a real model's proportions, in groups of three layers: differential attention (two
+    maps of half a head's size each), a chunked attention beside a gated delta rule, a state-space duality layer of twice
+    the width; every layer with the dense feed-forward."""
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "scale": (dim // 2) ** -0.5, "diff": 0.6,
+           "q_temp": {"coef": 0.1, "every": 1024}}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": chunk},
+            "rot": {"dims": dim // 2, "base": 1000000.0}}
+    right = {"heads": heads, "kv_heads": kv_heads, "dim": delta_dim, "vdim": dim, "conv": 4, "decay_rank": 32, "gate_rank": 32}
+    ssd = {"heads": 2 * width // ssd_dim, "vdim": ssd_dim, "state": ssd_state, "groups": ssd_groups, "norm_groups": ssd_groups, "conv": 4}
+    kinds = (("attention", att), ("parallel", {"left": left, "right": right}), ("mamba2", ssd))
+    return {"architecture": "Vagelix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "layers": [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+
+
+# Vagelix at the sizes of the Qwen2.5 shapes: the same width, heads, head size and dense feed-forward.
+DESIGN_PRESETS.update({
+    "vagelix-1.5b": _vagelix(151936, 1536, 27, 12, 2, 128, 8960),
+    "vagelix-7b": _vagelix(152064, 3584, 27, 28, 4, 128, 18944, ssd_groups=4),
+})
+
+
 def preset(name: str) -> Dict:
     import copy
     key = name.lower()

@@ -117,28 +117,56 @@ extern "C" int pico_ssd_prep(const void* bc, int ldb, int b_col, int c_col, int 
 // = ks * VC + vc holds S[ks * KPL .. ks * KPL + KPL - 1][v0 + vc].  The sums over key channels are added lane-locally in
 // channel order and then across the KS lanes of a column in a fixed tree: a token's output does not depend on how its
 // sequence was cut into steps or on what else the step holds.
+//
+// Long portions are cut into chunks of `chunk` tokens that run side by side.  A chunk maps the state in front of it to
+// the state behind it as S -> P S + L, with P [dk, dk] and L [dk, dv] that depend on the chunk's tokens alone:
+//   DS_LOCAL:  every chunk from a state of zero with its values: L.  With the delta rule P = prod_t (I - beta k k^T) diag(g)
+//              is no diagonal matrix; its column e is what the walk makes of the unit vector e with values of zero, so
+//              the same walk takes dk more columns (a state of [0 | I], values [v | 0]) and leaves [L | P].  Without the
+//              delta rule P is the product of the chunk's decays, a number a key channel.
+//   (delta_combine_kernel walks a sequence's chunks: ws_S[c] <- the state in front of chunk c, and the slot's final state)
+//   DS_FROM:   every chunk again from ws_S[chunk], writing the outputs
+// DS_WHOLE is the plain walk from the slot's state.  blockIdx.x = sequence * max_chunks + chunk in the chunked modes.
 // ---------------------------------------------------------------------------
-template <typename TV, int KPL, bool DELTA>
+#define DS_WHOLE 0
+#define DS_LOCAL 1
+#define DS_FROM 2
+
+template <typename TV, int KPL, bool DELTA, int MODE>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                         const TV* __restrict__ v, int ldv, const float* __restrict__ g,
                                                         int g_channels, const float* __restrict__ beta,
                                                         const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
                                                         float* __restrict__ state, float* __restrict__ out, int H, int KVH,
-                                                        int dk, int dv, int KS, int num_slots) {
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+                                                        int dk, int dv, int KS, int num_slots, int chunk, int max_chunks,
+                                                        float* __restrict__ ws_S, float* __restrict__ ws_P) {
+  const int b = MODE == DS_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, lane = threadIdx.x;
   const int VC = 64 / KS, vc = lane % VC, ks = lane / VC;
   const int col = blockIdx.z * VC + vc;
-  const int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1], slot = state_slots[b];
+  int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
+  if (MODE != DS_WHOLE) {
+    t_begin += (blockIdx.x % max_chunks) * chunk;
+    t_end = min(t_end, t_begin + chunk);
+  }
+  const int slot = state_slots[b];
   if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;
-  const bool col_ok = col < dv;
+  const int ncols = (MODE == DS_LOCAL && DELTA) ? dv + dk : dv;     // the unit vectors' columns behind the values'
+  const bool col_ok = col < ncols, unit = col >= dv;
   const int cin = min(col, dv - 1);
   const int c0 = ks * KPL;
   const int kvh = h / (H / KVH);
-  float* sp = state + (((size_t)slot * H + h) * dk) * dv + cin;
+  float* sp = MODE == DS_WHOLE ? state + (((size_t)slot * H + h) * dk) * dv + cin
+                               : ws_S + (((size_t)blockIdx.x * H + h) * dk) * dv + cin;
   float S[KPL];
 #pragma unroll
-  for (int i = 0; i < KPL; i++) S[i] = (c0 + i < dk) ? sp[(size_t)(c0 + i) * dv] : 0.f;
+  for (int i = 0; i < KPL; i++) {
+    if (MODE == DS_LOCAL) S[i] = (unit && c0 + i == col - dv) ? 1.f : 0.f;
+    else S[i] = (c0 + i < dk) ? sp[(size_t)(c0 + i) * dv] : 0.f;
+  }
   float kk[KPL], qq[KPL], gg[KPL], vv, bb;
+  float gprod[KPL];                                   // DS_LOCAL without the delta rule: the chunk's decays multiplied up
+#pragma unroll
+  for (int i = 0; i < KPL; i++) gprod[i] = 1.f;
   auto fetch = [&](int t) {
     const float* kr = k + ((size_t)t * KVH + kvh) * dk;
     const float* qr = q + ((size_t)t * KVH + kvh) * dk;
@@ -146,7 +174,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     for (int i = 0; i < KPL; i++) {
       const int c = min(c0 + i, dk - 1);
       kk[i] = kr[c];
-      qq[i] = qr[c];
+      qq[i] = MODE == DS_LOCAL ? 0.f : qr[c];
       gg[i] = g_channels ? g[((size_t)t * H + h) * dk + c] : 0.f;
     }
     if (!g_channels) {
@@ -158,6 +186,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     for (int i = 0; i < KPL; i++)
       if (c0 + i >= dk) { kk[i] = 0.f; qq[i] = 0.f; gg[i] = 1.f; }
     vv = load_f32(v + (size_t)t * ldv + (size_t)h * dv + cin);
+    if (MODE == DS_LOCAL && unit) vv = 0.f;
     bb = beta[(size_t)t * H + h];
   };
   fetch(t_begin);
@@ -179,7 +208,15 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
       u = bt * (vt - sk);
     } else {
 #pragma unroll
-      for (int i = 0; i < KPL; i++) S[i] *= gc[i];
+      for (int i = 0; i < KPL; i++) {
+        S[i] *= gc[i];
+        if (MODE == DS_LOCAL) gprod[i] *= gc[i];
+      }
+    }
+    if (MODE == DS_LOCAL) {
+#pragma unroll
+      for (int i = 0; i < KPL; i++) S[i] = fmaf(kc[i], u, S[i]);
+      continue;
     }
     float so = 0.f;
 #pragma unroll
@@ -190,22 +227,69 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     for (int o = VC; o < 64; o <<= 1) so += __shfl_xor(so, o);
     if (ks == 0 && col_ok) out[((size_t)t * H + h) * dv + col] = so;
   }
-  if (col_ok) {
+  if (MODE == DS_FROM || !col_ok) return;
+  if (MODE == DS_LOCAL && unit) {
+    float* pp = ws_P + (((size_t)blockIdx.x * H + h) * dk) * dk + (col - dv);
 #pragma unroll
     for (int i = 0; i < KPL; i++)
-      if (c0 + i < dk) sp[(size_t)(c0 + i) * dv] = S[i];
+      if (c0 + i < dk) pp[(size_t)(c0 + i) * dk] = S[i];
+    return;
   }
+#pragma unroll
+  for (int i = 0; i < KPL; i++)
+    if (c0 + i < dk) sp[(size_t)(c0 + i) * dv] = S[i];
+  if (MODE == DS_LOCAL && !DELTA && col == 0) {
+#pragma unroll
+    for (int i = 0; i < KPL; i++)
+      if (c0 + i < dk) ws_P[((size_t)blockIdx.x * H + h) * dk + c0 + i] = gprod[i];
+  }
+}
+
+// The walk over a sequence's chunks.  grid (sequences, heads, dv): a workgroup owns one value column, thread i its row:
+// ws_S[c][i][col] becomes the state in front of chunk c, the slot gets the state behind the last chunk.
+template <bool DELTA>
+__global__ __launch_bounds__(512) void delta_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                                                            float* __restrict__ state, float* __restrict__ ws_S,
+                                                            const float* __restrict__ ws_P, int H, int dk, int dv, int num_slots,
+                                                            int chunk, int max_chunks) {
+  extern __shared__ float sh[];           // [dk] the column of the state
+  const int b = blockIdx.x, h = blockIdx.y, col = blockIdx.z, i = threadIdx.x;
+  const int slot = state_slots[b], n = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || slot >= num_slots || n <= 0) return;
+  const bool row_ok = i < dk;
+  float* sp = state + (((size_t)slot * H + h) * dk + min(i, dk - 1)) * dv + col;
+  float s = row_ok ? *sp : 0.f;
+  const int chunks = (n + chunk - 1) / chunk;
+  for (int c = 0; c < chunks; c++) {
+    const size_t blk = (size_t)b * max_chunks + c;
+    float* lp = ws_S + ((blk * H + h) * dk + min(i, dk - 1)) * dv + col;
+    const float local = row_ok ? *lp : 0.f;
+    if (row_ok) *lp = s;                                 // the state in front of this chunk
+    if (DELTA) {
+      __syncthreads();
+      if (row_ok) sh[i] = s;
+      __syncthreads();
+      const float* pr = ws_P + ((blk * H + h) * dk + min(i, dk - 1)) * dk;
+      float acc = 0.f;
+      for (int e = 0; e < dk; e++) acc = fmaf(pr[e], sh[e], acc);
+      s = acc + local;
+    } else {
+      s = fmaf(ws_P[(blk * H + h) * dk + min(i, dk - 1)], s, local);
+    }
+  }
+  if (row_ok) *sp = s;
 }
 
 #define DELTA_MAX_KEY_DIM 512
 
 extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, int ldv, int v_dtype, const float* g,
                                int g_channels, const float* beta, const int* cu_seqlens, const int* state_slots, float* state,
-                               float* out, int num_seqs, int H, int KVH, int dk, int dv, int num_slots, int delta,
-                               hipStream_t stream) {
+                               float* out, int num_seqs, int H, int KVH, int dk, int dv, int num_slots, int delta, int chunk,
+                               int max_chunks, float* ws_S, float* ws_P, hipStream_t stream) {
   PICO_REQUIRE(num_seqs >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && dk > 0 && dk <= DELTA_MAX_KEY_DIM && dv > 0 && num_slots > 0,
                "pico_delta_scan: bad sizes (at most %d key channels a head)", DELTA_MAX_KEY_DIM);
   PICO_REQUIRE(ldv >= H * dv && H <= 65535, "pico_delta_scan: the rows do not hold the values");
+  PICO_REQUIRE(chunk >= 0 && (chunk == 0 || (max_chunks > 0 && ws_S && ws_P)), "pico_delta_scan: chunks need their workspace");
   if (num_seqs == 0) return 0;
   // key channels a lane: the fewest of 4, 8, 16, 32 with which at most 4 lanes share a column; beyond 128 channels
   // more lanes a column
@@ -214,29 +298,37 @@ extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, in
   int KS = 1;
   while (KS * kpl < dk) KS *= 2;
   const int VC = 64 / KS;
-  const dim3 grid(num_seqs, H, (dv + VC - 1) / VC);
-  PICO_REQUIRE(grid.z <= 65535, "pico_delta_scan: too many value channels");
-#define GO(TV, KPL)                                                                                                         \
-  do {                                                                                                                      \
-    if (delta)                                                                                                              \
-      delta_scan_kernel<TV, KPL, true><<<grid, 64, 0, stream>>>(q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens,    \
-                                                                state_slots, state, out, H, KVH, dk, dv, KS, num_slots);    \
-    else                                                                                                                    \
-      delta_scan_kernel<TV, KPL, false><<<grid, 64, 0, stream>>>(q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens,   \
-                                                                 state_slots, state, out, H, KVH, dk, dv, KS, num_slots);   \
+  const int cols_local = delta ? dv + dk : dv;
+  const dim3 grid_whole(num_seqs, H, (dv + VC - 1) / VC);
+  const dim3 grid_local((unsigned)(num_seqs * (chunk ? max_chunks : 1)), H, (cols_local + VC - 1) / VC);
+  const dim3 grid_from((unsigned)(num_seqs * (chunk ? max_chunks : 1)), H, (dv + VC - 1) / VC);
+  PICO_REQUIRE(grid_local.z <= 65535 && dv <= 65535, "pico_delta_scan: too many value channels");
+#define ARGS(TV) q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens, state_slots, state, out, H, KVH, dk, dv, KS, num_slots, \
+                 chunk, max_chunks, ws_S, ws_P
+#define GO(TV, KPL, D)                                                                            \
+  do {                                                                                            \
+    if (chunk == 0) {                                                                             \
+      delta_scan_kernel<TV, KPL, D, DS_WHOLE><<<grid_whole, 64, 0, stream>>>(ARGS(TV));           \
+    } else {                                                                                      \
+      delta_scan_kernel<TV, KPL, D, DS_LOCAL><<<grid_local, 64, 0, stream>>>(ARGS(TV));           \
+      delta_combine_kernel<D><<<dim3(num_seqs, H, dv), (dk + 63) / 64 * 64, dk * sizeof(float), stream>>>( \
+          cu_seqlens, state_slots, state, ws_S, ws_P, H, dk, dv, num_slots, chunk, max_chunks);   \
+      delta_scan_kernel<TV, KPL, D, DS_FROM><<<grid_from, 64, 0, stream>>>(ARGS(TV));             \
+    }                                                                                             \
   } while (0)
-#define PICK(TV)                    \
-  do {                              \
-    if (kpl == 4) GO(TV, 4);        \
-    else if (kpl == 8) GO(TV, 8);   \
-    else if (kpl == 16) GO(TV, 16); \
-    else GO(TV, 32);                \
+#define PICK(TV, D)                    \
+  do {                                 \
+    if (kpl == 4) GO(TV, 4, D);        \
+    else if (kpl == 8) GO(TV, 8, D);   \
+    else if (kpl == 16) GO(TV, 16, D); \
+    else GO(TV, 32, D);                \
   } while (0)
-  if (v_dtype == PICO_DTYPE_F32) PICK(float);
-  else if (v_dtype == PICO_DTYPE_BF16) PICK(bf16_t);
+  if (v_dtype == PICO_DTYPE_F32) { if (delta) PICK(float, true); else PICK(float, false); }
+  else if (v_dtype == PICO_DTYPE_BF16) { if (delta) PICK(bf16_t, true); else PICK(bf16_t, false); }
   else PICO_REQUIRE(false, "pico_delta_scan: unknown dtype %d", v_dtype);
 #undef PICK
 #undef GO
+#undef ARGS
   PICO_LAUNCH_CHECK();
   return 0;
 }

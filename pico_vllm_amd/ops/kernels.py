@@ -1391,12 +1391,15 @@ def ssd_prep(bc: torch.Tensor, b_col: int, c_col: int, n: int, y: torch.Tensor, 
 
 def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, cu_seqlens: torch.Tensor,
                state_slots: torch.Tensor, state: torch.Tensor, num_seqs: int, heads: int, kv_heads: int, dk: int, dv: int,
-               delta: bool = True) -> torch.Tensor:
+               delta: bool = True, chunk: int = 0) -> torch.Tensor:
     """The walk S <- diag(g_t) S; u = beta_t (v_t - S^T k_t) (``delta``; else u = beta_t v_t); S <- S + k_t u^T;
     o_t = S^T q_t, for every sequence of the step from its state slot (``state`` float32 [slots, heads, dk, dv], updated in
     place).  q, k float32 [T, kv_heads * dk] (head h reads q/k head h // (heads // kv_heads)); v [T, >= heads * dv] (row
     stride free); g float32 [T, heads * dk] (a decay a key channel) or [T, heads] (one a head); beta float32 [T, heads].
-    Returns o float32 [T, heads * dv]."""
+    Returns o float32 [T, heads * dv].
+    ``chunk`` > 0: sequences are cut into chunks of that many tokens that run side by side (every chunk from zero, which
+    also yields the chunk's map of the state in front of it; a walk over the chunks' states; every chunk again from its
+    true state): the same sums in another order."""
     _gpu(q, k, v, g, beta, cu_seqlens, state_slots, state)
     T = q.shape[0]
     for t, name in ((q, "q"), (k, "k")):
@@ -1416,10 +1419,17 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tenso
     _i32(cu_seqlens, "cu_seqlens", num_seqs + 1)
     _i32(state_slots, "state_slots", num_seqs)
     out = torch.empty(T, heads * dv, dtype=torch.float32, device=q.device)
+    ws_s = ws_p = None
+    max_chunks = 0
+    if chunk > 0:
+        max_chunks = -(-T // chunk)
+        ws_s = torch.empty(num_seqs * max_chunks, heads, dk, dv, dtype=torch.float32, device=q.device)
+        ws_p = torch.empty(num_seqs * max_chunks, heads, dk, dk if delta else 1, dtype=torch.float32, device=q.device)
     lib = library.core()
     _check(lib, lib.pico_delta_scan(_ptr(q), _ptr(k), _ptr(v), v.stride(0) if T > 1 else v.shape[1], _dt(v), _ptr(g),
                                     1 if g_channels else 0, _ptr(beta), _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out),
-                                    num_seqs, heads, kv_heads, dk, dv, state.shape[0], 1 if delta else 0, _stream()))
+                                    num_seqs, heads, kv_heads, dk, dv, state.shape[0], 1 if delta else 0, chunk, max_chunks, _ptr(ws_s),
+                                    _ptr(ws_p), _stream()))
     return out
 
 

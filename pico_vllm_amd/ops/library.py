@@ -158,7 +158,7 @@ def peaks() -> ctypes.CDLL:
 
 def build_all(head_dims: Iterable[int] = tuple(range(16, 257, 16)), force: bool = True,
               bias_dims: Iterable[tuple] = ((64, 32), (64, 64), (128, 64), (128, 128), (32, 16), (32, 64), (64, 48), (64, 16), (32, 32), (32, 96), (64, 96),
-                                          (128, 96), (64, 48), (96, 64), (320, 256), (256, 224), (288, 224))) -> List[str]:
+                                          (128, 96), (96, 64), (320, 256), (256, 224), (288, 224), (64, 128), (96, 96), (32, 48))) -> List[str]:
     """Compile everything (used by the build check); returns the paths."""
     out = [build_library("pico_core", CORE_SOURCES, force=force), build_library("pico_peaks", PEAK_SOURCES, force=force)]
     if os.path.isfile(os.path.join(CSRC, "attention_mfma.hip")):

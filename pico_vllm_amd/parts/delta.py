@@ -13,6 +13,16 @@ from .registry import register_part
 from .spec import CacheSpec, ParamSpec
 
 
+# In the bfloat16 engine a step with a prompt portion cuts its sequences into chunks of this many tokens that run side by
+# side (``kernels.delta_scan``); decided from the step's shape alone.  The 32-bit engine walks every sequence whole, so
+# that its sums do not depend on how a prompt was cut.
+CHUNK, CHUNKED_FROM = 64, 128
+
+
+def _chunk(act_dtype: torch.dtype, ctx: StepContext) -> int:
+    return CHUNK if act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= CHUNKED_FROM else 0
+
+
 def _conv_state(channels: int, taps: int) -> CacheSpec:
     """The last taps - 1 inputs of a short causal convolution, per channel."""
     return CacheSpec("state", state_shape=(channels, taps - 1), state_dtype="float32")
@@ -109,7 +119,7 @@ class GatedDeltaRule(Mixer):
         qn, kn, g, beta = kernels.delta_prep(xc, 0, self.k_col, y, self.b_col, self.a_col, self.a2, self.dt_bias, self.a_log,
                                              self.dk ** -0.5, self.heads, self.qk_heads, self.dk)
         o = kernels.delta_scan(qn, kn, xc[:, self.v_col:], g, beta, ctx.cu_seqlens, ctx.state_slots, state.state, ctx.num_seqs,
-                               self.heads, self.qk_heads, self.dk, self.dv, delta=True)
+                               self.heads, self.qk_heads, self.dk, self.dv, delta=True, chunk=_chunk(self.act_dtype, ctx))
         gate = self.g2(y[:, self.g_col:self.g_col + self.gate_rank])
         return kernels.gla_out(o, gate, 0, self.norm_weight, self.norm_eps, self.heads, self.dv, sigmoid_gate=True)
 
@@ -181,5 +191,5 @@ class StateSpaceDuality(Mixer):
         xbc = kernels.causal_conv(y[:, self.inner:], self.channels, self.conv_w, self.conv_b, ctx, hist.state, 0, single=ctx.all_decode)
         bf, cf, g, dt = kernels.ssd_prep(xbc, self.inner, self.inner + gn, gn, y, self.dt_col, self.dt_bias, self.a_log, self.heads)
         o = kernels.delta_scan(cf, bf, xbc, g, dt, ctx.cu_seqlens, ctx.state_slots, state.state, ctx.num_seqs, self.heads,
-                               self.groups, self.n, self.dv, delta=False)
+                               self.groups, self.n, self.dv, delta=False, chunk=_chunk(self.act_dtype, ctx))
         return kernels.gated_group_norm(o, xbc, y, self.d, self.norm_weight, self.norm_eps, self.heads, self.dv, self.norm_groups)

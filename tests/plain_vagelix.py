@@ -17,6 +17,25 @@ import torch
 
 F64 = torch.float64
 
+# A yardstick for what rounding alone does: with ``forward(..., rounding=f)`` every activation that passes from one part
+# to the next (a product's output, a convolution's, an attention's, the stream as a sublayer reads it) goes through f.
+_rounding = None
+
+
+def act(x: torch.Tensor) -> torch.Tensor:
+    return x if _rounding is None else _rounding(x)
+
+
+def stochastic_bfloat16(seed: int):
+    """A rounding to bfloat16's 8 significant bits that rounds up or down at random, in proportion (unbiased); draws
+    with different seeds are independent."""
+    g = torch.Generator().manual_seed(seed)
+
+    def f(x: torch.Tensor) -> torch.Tensor:
+        ulp = torch.exp2(torch.floor(torch.log2(x.abs().clamp_min(1e-300))) - 7)
+        return torch.floor(x / ulp + torch.rand(x.shape, generator=g, dtype=x.dtype)) * ulp
+    return f
+
 
 def rms(x: torch.Tensor, eps: float) -> torch.Tensor:
     """x over its root mean square along the last axis, eps inside the root."""
@@ -50,11 +69,11 @@ def differential_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict,
     q times the temperature of its position; causal softmax; o = a1 - lambda a2, over its root mean square, (1 - diff)."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ w["q"].T).view(T, H, 2, d)
-    k = (h @ w["k"].T).view(T, G, 2, d)
-    v = (h @ w["v"].T).view(T, G, dv)
-    q = rms(q, eps) * w["q.norm"]
-    k = rms(k, eps) * w["k.norm"]
+    q = act(h @ w["q"].T).view(T, H, 2, d)
+    k = act(h @ w["k"].T).view(T, G, 2, d)
+    v = act(h @ w["v"].T).view(T, G, dv)
+    q = act(rms(q, eps) * w["q.norm"])
+    k = act(rms(k, eps) * w["k.norm"])
     temp = torch.tensor([query_temperature(first_pos + t, m["q_temp"]["coef"], m["q_temp"]["every"]) if m.get("q_temp") else 1.0
                          for t in range(T)], dtype=h.dtype)
     q = q * temp.view(T, 1, 1, 1)
@@ -70,7 +89,7 @@ def differential_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict,
             maps.append(torch.softmax(s, dim=-1) @ v[:, g])
         o = maps[0] - lam * maps[1]
         out[:, hh] = rms(o, eps) * (1.0 - m["diff"])
-    return out.reshape(T, H * dv) @ w["o"].T
+    return act(act(out.reshape(T, H * dv)) @ w["o"].T)
 
 
 # ---- the parallel mixer's left side: chunked attention with a sink ---------------------------------------------------
@@ -96,19 +115,19 @@ def chunked_sink_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict,
     j <= i of its own chunk; p_j = exp(s_j) / (1 + sum exp(s)); head outputs times sigmoid(Wg h), one number a head."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = h @ w["q"].T + w["q.b"]
-    k = h @ w["k"].T + w["k.b"]
+    q = act(h @ w["q"].T + w["q.b"])
+    k = act(h @ w["k"].T + w["k.b"])
     v = k.view(T, G, d)
     assert dv == d, "the values are the keys: their sizes are one"
     q = (rms(q, eps) * w["q.norm"]).view(T, H, d)
     kn = (rms(k, eps) * w["k.norm"]).view(T, G, d)
     pos = torch.arange(first_pos, first_pos + T)
     rot = m.get("rot") or {}
-    q = rotate_half(q, pos, rot.get("dims", 0), rot.get("base", 1.0))
-    kn = rotate_half(kn, pos, rot.get("dims", 0), rot.get("base", 1.0))
+    q = act(rotate_half(q, pos, rot.get("dims", 0), rot.get("base", 1.0)))
+    kn = act(rotate_half(kn, pos, rot.get("dims", 0), rot.get("base", 1.0)))
     size = (m.get("mask") or {}).get("size", 0)
     vis = torch.tensor([[chunk_visible(first_pos + i, first_pos + j, size) for j in range(T)] for i in range(T)])
-    gate = torch.sigmoid(h @ w["g"].T)                                  # [T, H]
+    gate = torch.sigmoid(act(h @ w["g"].T))                             # [T, H]
     out = torch.zeros(T, H, dv, dtype=h.dtype)
     for hh in range(H):
         g = kv_head_of(hh, H, G)
@@ -116,7 +135,7 @@ def chunked_sink_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict,
         e = torch.where(vis, torch.exp(s), torch.zeros_like(s))
         p = e / (1.0 + e.sum(-1, keepdim=True))
         out[:, hh] = (p @ v[:, g]) * gate[:, hh:hh + 1]
-    return out.reshape(T, H * dv) @ w["o"].T
+    return act(act(out.reshape(T, H * dv)) @ w["o"].T)
 
 
 # ---- short causal convolution ----------------------------------------------------------------------------------------
@@ -153,21 +172,21 @@ def delta_rule_scan(q, k, v, g, beta, S0=None):
 def gated_delta_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float) -> torch.Tensor:
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = silu(causal_conv(h @ w["q"].T, w["q.conv"])).view(T, G, dk)
-    k = silu(causal_conv(h @ w["k"].T, w["k.conv"])).view(T, G, dk)
-    v = silu(causal_conv(h @ w["v"].T, w["v.conv"])).view(T, H, dv)
+    q = act(silu(causal_conv(act(h @ w["q"].T), w["q.conv"]))).view(T, G, dk)
+    k = act(silu(causal_conv(act(h @ w["k"].T), w["k.conv"]))).view(T, G, dk)
+    v = act(silu(causal_conv(act(h @ w["v"].T), w["v.conv"]))).view(T, H, dv)
     unit = lambda x: x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
     q = unit(q) * dk ** -0.5
     k = unit(k)
     idx = torch.tensor([kv_head_of(i, H, G) for i in range(H)])
     q, k = q[:, idx], k[:, idx]
-    beta = torch.sigmoid(h @ w["b"].T)                                                    # [T, H]
-    step = softplus((h @ w["a1"].T) @ w["a2"].T + w["dt_bias"]).view(T, H, dk)
+    beta = torch.sigmoid(act(h @ w["b"].T))                                               # [T, H]
+    step = softplus(act(h @ w["a1"].T) @ w["a2"].T + w["dt_bias"]).view(T, H, dk)
     g = torch.exp(-torch.exp(w["A_log"]).view(1, H, 1) * step)
     o, _ = delta_rule_scan(q, k, v, g, beta)
     o = rms(o, eps) * w["norm"]
-    o = o * torch.sigmoid((h @ w["g1"].T) @ w["g2"].T).view(T, H, dv)
-    return o.reshape(T, H * dv) @ w["o"].T
+    o = o * torch.sigmoid(act(act(h @ w["g1"].T) @ w["g2"].T)).view(T, H, dv)
+    return act(act(o.reshape(T, H * dv)) @ w["o"].T)
 
 
 def parallel_mixer(h, w, m, eps, first_pos: int = 0):
@@ -196,9 +215,9 @@ def mamba2_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: floa
     T = h.shape[0]
     H, dv, N, G, ng = m["heads"], m["vdim"], m["state"], m["groups"], m["norm_groups"]
     inner = H * dv
-    y = h @ w["in"].T
+    y = act(h @ w["in"].T)
     z, xbc, dt = y[:, :inner], y[:, inner:2 * inner + 2 * G * N], y[:, 2 * inner + 2 * G * N:]
-    xbc = silu(causal_conv(xbc, w["conv"], w["conv.b"]))
+    xbc = act(silu(causal_conv(xbc, w["conv"], w["conv.b"])))
     x = xbc[:, :inner].view(T, H, dv)
     B = xbc[:, inner:inner + G * N].view(T, G, N)
     C = xbc[:, inner + G * N:].view(T, G, N)
@@ -207,12 +226,12 @@ def mamba2_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: floa
     yy, _ = ssd_scan(x, B[:, idx], C[:, idx], dt, torch.exp(w["A_log"]), w["D"])
     yy = yy.reshape(T, inner) * silu(z)
     yy = rms(yy.view(T, ng, inner // ng), eps).reshape(T, inner) * w["norm"]
-    return yy @ w["o"].T
+    return act(act(yy) @ w["o"].T)
 
 
 # ---- feed-forward, layers, model -------------------------------------------------------------------------------------
 def dense_mlp(h, w):
-    return (silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
+    return act(act(silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T)
 
 
 def weight_owner(layers: List[dict], i: int) -> int:
@@ -221,8 +240,20 @@ def weight_owner(layers: List[dict], i: int) -> int:
     return i
 
 
-def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=F64, trace: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence from position 0.  ``trace``: a list that receives the stream after every layer."""
+def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=F64, trace: Optional[list] = None,
+            rounding=None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence from position 0.  ``trace``: a list that receives the stream after every layer.
+    ``rounding``: a function that every activation between the parts goes through (the stream itself stays as it is; what
+    a sublayer reads of it is rounded)."""
+    global _rounding
+    _rounding = rounding
+    try:
+        return _forward(cfg, weights, tokens, dtype, trace)
+    finally:
+        _rounding = None
+
+
+def _forward(cfg, weights, tokens, dtype, trace):
     W = {n: (t.to(dtype) if t.is_floating_point() else t) for n, t in weights.items()}
     eps = cfg["norm"]["eps"]
     x = rms(W["embed"][torch.tensor(tokens)], eps) * W["embed.norm"]
@@ -232,16 +263,77 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
         mw = {n[4:]: t for n, t in lw.items() if n.startswith("mix.")}
         kind, m = layer["type"], layer["mixer"]
         if kind == "attention":
-            y = differential_attention(x, mw, m, eps)
+            y = differential_attention(act(x), mw, m, eps)
         elif kind == "parallel":
-            y = parallel_mixer(x, mw, m, eps)
+            y = parallel_mixer(act(x), mw, m, eps)
         elif kind == "mamba2":
-            y = mamba2_mixer(x, mw, m, eps)
+            y = mamba2_mixer(act(x), mw, m, eps)
         else:
             raise ValueError(f"unknown mixer {kind!r}")
         x = x + rms(y, eps) * lw["norm1"]
         if layer.get("mlp"):
-            x = x + rms(dense_mlp(x, {n[4:]: t for n, t in lw.items() if n.startswith("mlp.")}), eps) * lw["norm2"]
+            x = x + rms(dense_mlp(act(x), {n[4:]: t for n, t in lw.items() if n.startswith("mlp.")}), eps) * lw["norm2"]
         if trace is not None:
             trace.append(x.clone())
-    return (rms(x, eps) * W["final.norm"]) @ W["embed"].T
+    return act(rms(x, eps) * W["final.norm"]) @ W["embed"].T
+
+
+# ---- random models -----------------------------------------------------------------------------------------------------
+def tensor_shapes(cfg: dict, decay_rank: int = 6, gate_rank: int = 5) -> Dict[str, tuple]:
+    """Name -> shape of every tensor a model of this configuration holds (layers with weights_of hold none)."""
+    D, V = cfg["width"], cfg["vocab"]
+    out = {"embed": (V, D), "embed.norm": (D,), "final.norm": (D,)}
+    for i, layer in enumerate(cfg["layers"]):
+        if layer.get("weights_of") is not None:
+            continue
+        p, m = f"l{i}.", layer["mixer"]
+        out[p + "norm1"] = (D,)
+        if layer["type"] == "attention":
+            H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out.update({p + "mix.q": (H * 2 * d, D), p + "mix.k": (G * 2 * d, D), p + "mix.v": (G * dv, D), p + "mix.o": (D, H * dv),
+                        p + "mix.q.norm": (d,), p + "mix.k.norm": (d,)})
+            out.update({p + "mix." + n: (d,) for n in ("lq1", "lk1", "lq2", "lk2")})
+        elif layer["type"] == "parallel":
+            a, r = m["left"], m["right"]
+            H, G, d = a["heads"], a["kv_heads"], a["dim"]
+            q = p + "mix.left."
+            out.update({q + "q": (H * d, D), q + "q.b": (H * d,), q + "k": (G * d, D), q + "k.b": (G * d,), q + "q.norm": (H * d,),
+                        q + "k.norm": (G * d,), q + "g": (H, D), q + "o": (D, H * d), q + "out": (D,)})
+            H, G, d, dv, K = r["heads"], r["kv_heads"], r["dim"], r["vdim"], r["conv"]
+            q = p + "mix.right."
+            out.update({q + "q": (G * d, D), q + "q.conv": (G * d, K), q + "k": (G * d, D), q + "k.conv": (G * d, K),
+                        q + "v": (H * dv, D), q + "v.conv": (H * dv, K), q + "b": (H, D), q + "A_log": (H,), q + "norm": (dv,),
+                        q + "a1": (decay_rank, D), q + "a2": (H * d, decay_rank), q + "dt_bias": (H * d,),
+                        q + "g1": (gate_rank, D), q + "g2": (H * dv, gate_rank), q + "o": (D, H * dv), q + "out": (D,)})
+        else:
+            H, dv, N, G, K = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
+            inner, C = H * dv, H * dv + 2 * G * N
+            out.update({p + "mix.in": (inner + C + H, D), p + "mix.conv": (C, K), p + "mix.conv.b": (C,), p + "mix.dt_bias": (H,),
+                        p + "mix.A_log": (H,), p + "mix.D": (H,), p + "mix.norm": (inner,), p + "mix.o": (D, inner)})
+        if layer.get("mlp"):
+            F = layer["mlp"]["ff"]
+            out.update({p + "norm2": (D,), p + "mlp.gate": (F, D), p + "mlp.up": (F, D), p + "mlp.down": (D, F)})
+    return out
+
+
+def random_model(cfg: dict, seed: int, decay_rank: int = 6, gate_rank: int = 5) -> Dict[str, torch.Tensor]:
+    """Random bfloat16 tensors for ``cfg``: matrices N(0, 1 / sqrt(in)), norm weights around 1, what enters a recurrence
+    of a size that makes decays and gates neither 0 nor 1."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg, decay_rank, gate_rank).items():
+        last = name.rsplit(".", 1)[-1]
+        if last in ("norm", "norm1", "norm2", "out") or name in ("embed.norm", "final.norm"):
+            t = 1.0 + 0.3 * (2 * torch.rand(shape, generator=g) - 1)
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            t = 0.3 * torch.randn(shape, generator=g)
+        elif last == "conv":
+            t = 0.6 * torch.randn(shape, generator=g)
+        elif last in ("A_log", "dt_bias", "D", "b") and len(shape) == 1:
+            t = 0.7 * torch.randn(shape, generator=g)
+        elif name == "embed":
+            t = torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) * (1.5 / math.sqrt(shape[-1]))
+        out[name] = t.to(torch.bfloat16)
+    return out
