@@ -113,10 +113,14 @@ extern "C" int pico_ssd_prep(const void* bc, int ldb, int b_col, int c_col, int 
 }
 
 // ---------------------------------------------------------------------------
-// The walk.  grid (sequences, heads, ceil(dv / VC)), one wave a workgroup; VC = 64 / KS value columns a wave; lane
-// = ks * VC + vc holds S[ks * KPL .. ks * KPL + KPL - 1][v0 + vc].  The sums over key channels are added lane-locally in
-// channel order and then across the KS lanes of a column in a fixed tree: a token's output does not depend on how its
-// sequence was cut into steps or on what else the step holds.
+// The walk.  grid (sequences, heads, column tiles); a workgroup of up to four waves owns a tile of value columns of one
+// head of one sequence.  In a wave VC = 64 / KS lanes stand side by side over columns and KS lanes share a column, each
+// with KPL of its key channels; a lane owns VPL columns (VC apart), so what it reads of a token's k, g and q serves them
+// all: a thread keeps KPL * VPL state elements in registers for the whole step.  Tokens are taken TB at a time: their k,
+// q, decays, beta and the tile's values are staged in LDS by the whole workgroup (every load unconditional, from a
+// clamped address).  The sums over key channels are added lane-locally in channel order and then across the KS lanes
+// of a column in a fixed tree: a token's output does not depend on how its sequence was cut into steps or on what else
+// the step holds.
 //
 // Long portions are cut into chunks of `chunk` tokens that run side by side.  A chunk maps the state in front of it to
 // the state behind it as S -> P S + L, with P [dk, dk] and L [dk, dv] that depend on the chunk's tokens alone:
@@ -124,7 +128,7 @@ extern "C" int pico_ssd_prep(const void* bc, int ldb, int b_col, int c_col, int 
 //              is no diagonal matrix; its column e is what the walk makes of the unit vector e with values of zero, so
 //              the same walk takes dk more columns (a state of [0 | I], values [v | 0]) and leaves [L | P].  Without the
 //              delta rule P is the product of the chunk's decays, a number a key channel.
-//   (delta_combine_kernel walks a sequence's chunks: ws_S[c] <- the state in front of chunk c, and the slot's final state)
+//   (the combine kernels walk a sequence's chunks: ws_S[c] <- the state in front of chunk c, and the slot's final state)
 //   DS_FROM:   every chunk again from ws_S[chunk], writing the outputs
 // DS_WHOLE is the plain walk from the slot's state.  blockIdx.x = sequence * max_chunks + chunk in the chunked modes.
 // ---------------------------------------------------------------------------
@@ -132,152 +136,252 @@ extern "C" int pico_ssd_prep(const void* bc, int ldb, int b_col, int c_col, int 
 #define DS_LOCAL 1
 #define DS_FROM 2
 
-template <typename TV, int KPL, bool DELTA, int MODE>
-__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ q, const float* __restrict__ k,
-                                                        const TV* __restrict__ v, int ldv, const float* __restrict__ g,
-                                                        int g_channels, const float* __restrict__ beta,
-                                                        const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
-                                                        float* __restrict__ state, float* __restrict__ out, int H, int KVH,
-                                                        int dk, int dv, int KS, int num_slots, int chunk, int max_chunks,
-                                                        float* __restrict__ ws_S, float* __restrict__ ws_P) {
-  const int b = MODE == DS_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y, lane = threadIdx.x;
+template <typename TV, int KPL, int VPL, bool DELTA, int MODE>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                         const TV* __restrict__ v, int ldv, const float* __restrict__ g,
+                                                         int g_channels, const float* __restrict__ beta,
+                                                         const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                                                         float* __restrict__ state, float* __restrict__ out, int H, int KVH,
+                                                         int dk, int dv, int KS, int TB, int num_slots, int chunk,
+                                                         int max_chunks, float* __restrict__ ws_S, float* __restrict__ ws_P) {
+  extern __shared__ float lds[];
+  const int b = MODE == DS_WHOLE ? blockIdx.x : blockIdx.x / max_chunks, h = blockIdx.y;
+  const int nw = blockDim.x >> 6, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int VC = 64 / KS, vc = lane % VC, ks = lane / VC;
-  const int col = blockIdx.z * VC + vc;
+  const int DKP = KS * KPL;                            // key channels with padding
+  const int tile = nw * VC * VPL;                      // columns of the workgroup
+  float* ks_ = lds;                                    // [TB][DKP]
+  float* qs_ = ks_ + TB * DKP;
+  float* gs_ = qs_ + TB * DKP;
+  float* vs_ = gs_ + TB * DKP;                         // [TB][tile]
+  float* bs_ = vs_ + TB * tile;                        // [TB]
   int t_begin = cu_seqlens[b], t_end = cu_seqlens[b + 1];
   if (MODE != DS_WHOLE) {
     t_begin += (blockIdx.x % max_chunks) * chunk;
     t_end = min(t_end, t_begin + chunk);
   }
   const int slot = state_slots[b];
-  if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;
-  const int ncols = (MODE == DS_LOCAL && DELTA) ? dv + dk : dv;     // the unit vectors' columns behind the values'
-  const bool col_ok = col < ncols, unit = col >= dv;
-  const int cin = min(col, dv - 1);
+  if (slot < 0 || slot >= num_slots || t_end <= t_begin) return;          // the whole workgroup
+  const int ncols = (MODE == DS_LOCAL && DELTA) ? dv + dk : dv;           // the unit vectors' columns behind the values'
+  const int col0 = blockIdx.z * tile, lcol0 = wave * VC * VPL + vc;       // the tile's first column; this lane's first in the tile
   const int c0 = ks * KPL;
   const int kvh = h / (H / KVH);
-  float* sp = MODE == DS_WHOLE ? state + (((size_t)slot * H + h) * dk) * dv + cin
-                               : ws_S + (((size_t)blockIdx.x * H + h) * dk) * dv + cin;
-  float S[KPL];
+  float* sbase = MODE == DS_WHOLE ? state + (((size_t)slot * H + h) * dk) * dv
+                                  : ws_S + (((size_t)blockIdx.x * H + h) * dk) * dv;
+  float S[VPL][KPL];
 #pragma unroll
-  for (int i = 0; i < KPL; i++) {
-    if (MODE == DS_LOCAL) S[i] = (unit && c0 + i == col - dv) ? 1.f : 0.f;
-    else S[i] = (c0 + i < dk) ? sp[(size_t)(c0 + i) * dv] : 0.f;
+  for (int j = 0; j < VPL; j++) {
+    const int col = col0 + lcol0 + j * VC;
+#pragma unroll
+    for (int i = 0; i < KPL; i++) {
+      if (MODE == DS_LOCAL) S[j][i] = (col >= dv && col < ncols && c0 + i == col - dv) ? 1.f : 0.f;
+      else {
+        const float x = sbase[(size_t)min(c0 + i, dk - 1) * dv + min(col, dv - 1)];
+        S[j][i] = (c0 + i < dk && col < dv) ? x : 0.f;
+      }
+    }
   }
-  float kk[KPL], qq[KPL], gg[KPL], vv, bb;
-  float gprod[KPL];                                   // DS_LOCAL without the delta rule: the chunk's decays multiplied up
+  float gprod[KPL];                                    // DS_LOCAL without the delta rule: the chunk's decays multiplied up
 #pragma unroll
   for (int i = 0; i < KPL; i++) gprod[i] = 1.f;
-  auto fetch = [&](int t) {
-    const float* kr = k + ((size_t)t * KVH + kvh) * dk;
-    const float* qr = q + ((size_t)t * KVH + kvh) * dk;
-#pragma unroll
-    for (int i = 0; i < KPL; i++) {
-      const int c = min(c0 + i, dk - 1);
-      kk[i] = kr[c];
-      qq[i] = MODE == DS_LOCAL ? 0.f : qr[c];
-      gg[i] = g_channels ? g[((size_t)t * H + h) * dk + c] : 0.f;
+  for (int t0 = t_begin; t0 < t_end; t0 += TB) {
+    const int nb = min(TB, t_end - t0);
+    __syncthreads();                                   // the last block's staged values have been read
+    for (int idx = threadIdx.x; idx < nb * DKP; idx += blockDim.x) {      // only the block's tokens: a single token is one turn
+      const int tt = idx / DKP, c = idx % DKP;
+      const int t = t0 + min(tt, nb - 1), cc = min(c, dk - 1);
+      const bool in = tt < nb && c < dk;
+      const float kx = k[((size_t)t * KVH + kvh) * dk + cc];
+      const float qx = MODE == DS_LOCAL ? 0.f : q[((size_t)t * KVH + kvh) * dk + cc];
+      const float gx = g_channels ? g[((size_t)t * H + h) * dk + cc] : g[(size_t)t * H + h];
+      ks_[idx] = in ? kx : 0.f;
+      qs_[idx] = in ? qx : 0.f;
+      gs_[idx] = in ? gx : 1.f;
     }
-    if (!g_channels) {
-      const float gh = g[(size_t)t * H + h];
-#pragma unroll
-      for (int i = 0; i < KPL; i++) gg[i] = gh;
+    for (int idx = threadIdx.x; idx < nb * tile; idx += blockDim.x) {
+      const int tt = idx / tile, col = col0 + idx % tile;
+      const float x = load_f32(v + (size_t)(t0 + min(tt, nb - 1)) * ldv + (size_t)h * dv + min(col, dv - 1));
+      vs_[idx] = (tt < nb && col < dv) ? x : 0.f;       // the unit vectors' columns have values of zero
     }
+    if ((int)threadIdx.x < TB) bs_[threadIdx.x] = beta[(size_t)(t0 + min((int)threadIdx.x, nb - 1)) * H + h];
+    __syncthreads();
+    for (int tt = 0; tt < nb; tt++) {
+      const float4* k4 = reinterpret_cast<const float4*>(ks_ + tt * DKP + c0);
+      const float4* g4 = reinterpret_cast<const float4*>(gs_ + tt * DKP + c0);
+      const float4* q4 = reinterpret_cast<const float4*>(qs_ + tt * DKP + c0);
+      const float bt = bs_[tt];
+      float kc[KPL], u[VPL];
 #pragma unroll
-    for (int i = 0; i < KPL; i++)
-      if (c0 + i >= dk) { kk[i] = 0.f; qq[i] = 0.f; gg[i] = 1.f; }
-    vv = load_f32(v + (size_t)t * ldv + (size_t)h * dv + cin);
-    if (MODE == DS_LOCAL && unit) vv = 0.f;
-    bb = beta[(size_t)t * H + h];
-  };
-  fetch(t_begin);
-  for (int t = t_begin; t < t_end; t++) {
-    float kc[KPL], qc[KPL], gc[KPL];
+      for (int j = 0; j < VPL; j++) u[j] = 0.f;
 #pragma unroll
-    for (int i = 0; i < KPL; i++) { kc[i] = kk[i]; qc[i] = qq[i]; gc[i] = gg[i]; }
-    const float vt = vv, bt = bb;
-    if (t + 1 < t_end) fetch(t + 1);                     // the next token's operands travel while this one is worked on
-    float u = bt * vt;
-    if (DELTA) {
-      float sk = 0.f;
+      for (int i = 0; i < KPL / 4; i++) {
+        const float4 kv = k4[i], gv = g4[i];
+        kc[4 * i] = kv.x; kc[4 * i + 1] = kv.y; kc[4 * i + 2] = kv.z; kc[4 * i + 3] = kv.w;
+        if (MODE == DS_LOCAL && !DELTA) { gprod[4 * i] *= gv.x; gprod[4 * i + 1] *= gv.y; gprod[4 * i + 2] *= gv.z; gprod[4 * i + 3] *= gv.w; }
 #pragma unroll
-      for (int i = 0; i < KPL; i++) {
-        S[i] *= gc[i];
-        sk = fmaf(S[i], kc[i], sk);
+        for (int j = 0; j < VPL; j++) {
+          S[j][4 * i] *= gv.x; S[j][4 * i + 1] *= gv.y; S[j][4 * i + 2] *= gv.z; S[j][4 * i + 3] *= gv.w;
+          if (DELTA) {
+            u[j] = fmaf(S[j][4 * i], kv.x, u[j]); u[j] = fmaf(S[j][4 * i + 1], kv.y, u[j]);
+            u[j] = fmaf(S[j][4 * i + 2], kv.z, u[j]); u[j] = fmaf(S[j][4 * i + 3], kv.w, u[j]);
+          }
+        }
       }
-      for (int o = VC; o < 64; o <<= 1) sk += __shfl_xor(sk, o);
-      u = bt * (vt - sk);
-    } else {
 #pragma unroll
-      for (int i = 0; i < KPL; i++) {
-        S[i] *= gc[i];
-        if (MODE == DS_LOCAL) gprod[i] *= gc[i];
+      for (int j = 0; j < VPL; j++) {
+        const float vt = vs_[tt * tile + lcol0 + j * VC];
+        if (DELTA) {
+          float sk = u[j];
+          for (int o = VC; o < 64; o <<= 1) sk += __shfl_xor(sk, o);
+          u[j] = bt * (vt - sk);
+        } else {
+          u[j] = bt * vt;
+        }
+      }
+      if (MODE == DS_LOCAL) {
+#pragma unroll
+        for (int j = 0; j < VPL; j++)
+#pragma unroll
+          for (int i = 0; i < KPL; i++) S[j][i] = fmaf(kc[i], u[j], S[j][i]);
+        continue;
+      }
+      float so[VPL];
+#pragma unroll
+      for (int j = 0; j < VPL; j++) so[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < KPL / 4; i++) {
+        const float4 qv = q4[i];
+#pragma unroll
+        for (int j = 0; j < VPL; j++) {
+          S[j][4 * i] = fmaf(kc[4 * i], u[j], S[j][4 * i]); so[j] = fmaf(S[j][4 * i], qv.x, so[j]);
+          S[j][4 * i + 1] = fmaf(kc[4 * i + 1], u[j], S[j][4 * i + 1]); so[j] = fmaf(S[j][4 * i + 1], qv.y, so[j]);
+          S[j][4 * i + 2] = fmaf(kc[4 * i + 2], u[j], S[j][4 * i + 2]); so[j] = fmaf(S[j][4 * i + 2], qv.z, so[j]);
+          S[j][4 * i + 3] = fmaf(kc[4 * i + 3], u[j], S[j][4 * i + 3]); so[j] = fmaf(S[j][4 * i + 3], qv.w, so[j]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < VPL; j++) {
+        float x = so[j];
+        for (int o = VC; o < 64; o <<= 1) x += __shfl_xor(x, o);
+        const int col = col0 + lcol0 + j * VC;
+        if (ks == 0 && col < dv) out[((size_t)(t0 + tt) * H + h) * dv + col] = x;
       }
     }
-    if (MODE == DS_LOCAL) {
+  }
+  if (MODE == DS_FROM) return;
 #pragma unroll
-      for (int i = 0; i < KPL; i++) S[i] = fmaf(kc[i], u, S[i]);
+  for (int j = 0; j < VPL; j++) {
+    const int col = col0 + lcol0 + j * VC;
+    if (col >= ncols) continue;
+    if (col >= dv) {                                   // DS_LOCAL with the delta rule: column col - dv of P
+      float* pp = ws_P + (((size_t)blockIdx.x * H + h) * dk) * dk + (col - dv);
+#pragma unroll
+      for (int i = 0; i < KPL; i++)
+        if (c0 + i < dk) pp[(size_t)(c0 + i) * dk] = S[j][i];
       continue;
     }
-    float so = 0.f;
 #pragma unroll
-    for (int i = 0; i < KPL; i++) {
-      S[i] = fmaf(kc[i], u, S[i]);
-      so = fmaf(S[i], qc[i], so);
+    for (int i = 0; i < KPL; i++)
+      if (c0 + i < dk) sbase[(size_t)(c0 + i) * dv + col] = S[j][i];
+    if (MODE == DS_LOCAL && !DELTA && col == 0) {
+#pragma unroll
+      for (int i = 0; i < KPL; i++)
+        if (c0 + i < dk) ws_P[((size_t)blockIdx.x * H + h) * dk + c0 + i] = gprod[i];
     }
-    for (int o = VC; o < 64; o <<= 1) so += __shfl_xor(so, o);
-    if (ks == 0 && col_ok) out[((size_t)t * H + h) * dv + col] = so;
-  }
-  if (MODE == DS_FROM || !col_ok) return;
-  if (MODE == DS_LOCAL && unit) {
-    float* pp = ws_P + (((size_t)blockIdx.x * H + h) * dk) * dk + (col - dv);
-#pragma unroll
-    for (int i = 0; i < KPL; i++)
-      if (c0 + i < dk) pp[(size_t)(c0 + i) * dk] = S[i];
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < KPL; i++)
-    if (c0 + i < dk) sp[(size_t)(c0 + i) * dv] = S[i];
-  if (MODE == DS_LOCAL && !DELTA && col == 0) {
-#pragma unroll
-    for (int i = 0; i < KPL; i++)
-      if (c0 + i < dk) ws_P[((size_t)blockIdx.x * H + h) * dk + c0 + i] = gprod[i];
   }
 }
 
-// The walk over a sequence's chunks.  grid (sequences, heads, dv): a workgroup owns one value column, thread i its row:
-// ws_S[c][i][col] becomes the state in front of chunk c, the slot gets the state behind the last chunk.
-template <bool DELTA>
-__global__ __launch_bounds__(512) void delta_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+// The walk over a sequence's chunks without the delta rule, one thread per state element: ws_S[c] becomes the state in
+// front of chunk c, the slot gets the state behind the last chunk.  grid (sequences, heads, ceil(dk dv / 256)).
+__global__ __launch_bounds__(256) void decay_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
                                                             float* __restrict__ state, float* __restrict__ ws_S,
                                                             const float* __restrict__ ws_P, int H, int dk, int dv, int num_slots,
                                                             int chunk, int max_chunks) {
-  extern __shared__ float sh[];           // [dk] the column of the state
-  const int b = blockIdx.x, h = blockIdx.y, col = blockIdx.z, i = threadIdx.x;
+  const int b = blockIdx.x, h = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= dk * dv) return;
   const int slot = state_slots[b], n = cu_seqlens[b + 1] - cu_seqlens[b];
   if (slot < 0 || slot >= num_slots || n <= 0) return;
-  const bool row_ok = i < dk;
-  float* sp = state + (((size_t)slot * H + h) * dk + min(i, dk - 1)) * dv + col;
-  float s = row_ok ? *sp : 0.f;
+  const int i = e / dv;
+  float* sp = state + ((size_t)slot * H + h) * dk * dv + e;
+  float s = *sp;
   const int chunks = (n + chunk - 1) / chunk;
   for (int c = 0; c < chunks; c++) {
     const size_t blk = (size_t)b * max_chunks + c;
-    float* lp = ws_S + ((blk * H + h) * dk + min(i, dk - 1)) * dv + col;
-    const float local = row_ok ? *lp : 0.f;
-    if (row_ok) *lp = s;                                 // the state in front of this chunk
-    if (DELTA) {
-      __syncthreads();
-      if (row_ok) sh[i] = s;
-      __syncthreads();
-      const float* pr = ws_P + ((blk * H + h) * dk + min(i, dk - 1)) * dk;
-      float acc = 0.f;
-      for (int e = 0; e < dk; e++) acc = fmaf(pr[e], sh[e], acc);
-      s = acc + local;
-    } else {
-      s = fmaf(ws_P[(blk * H + h) * dk + min(i, dk - 1)], s, local);
-    }
+    float* lp = ws_S + (blk * H + h) * dk * dv + e;
+    const float local = *lp, p = ws_P[(blk * H + h) * dk + i];
+    *lp = s;
+    s = fmaf(p, s, local);
   }
-  if (row_ok) *sp = s;
+  *sp = s;
+}
+
+// The same with the delta rule: S <- P S + L with a full matrix P [dk, dk] a chunk.  grid (sequences, heads,
+// ceil(dv / 16)); a workgroup of 256 threads owns 16 value columns, thread (r, j) the rows r, r + 16, .. of column j.
+// The tile of the state and, ET columns at a time, the chunk's P stand in LDS for the products (P is read from memory
+// once a workgroup, in rows' order).
+#define DC_ROWS 32          // rows a thread: 512 key channels at most
+__global__ __launch_bounds__(256) void delta_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                                                            float* __restrict__ state, float* __restrict__ ws_S,
+                                                            const float* __restrict__ ws_P, int H, int dk, int dv, int num_slots,
+                                                            int chunk, int max_chunks, int ET) {
+  extern __shared__ float sh[];           // [dk + 3][16] the state's tile (three rows of zeros behind it), then [dk][ET] of P
+  float* pt = sh + (dk + 3) * 16;          // ET is a multiple of 4: the columns behind the last of P hold zeros
+  if (threadIdx.x < 48) sh[dk * 16 + threadIdx.x] = 0.f;
+  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x & 15, r = threadIdx.x >> 4;
+  const int col = blockIdx.z * 16 + j, cin = min(col, dv - 1);
+  const int slot = state_slots[b], n = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || slot >= num_slots || n <= 0) return;          // the whole workgroup
+  const int rows = (dk - r + 15) / 16;                          // rows r, r + 16, .. below dk
+  float s[DC_ROWS], acc[DC_ROWS];
+  float* sp = state + ((size_t)slot * H + h) * dk * dv + cin;
+#pragma unroll
+  for (int x = 0; x < DC_ROWS; x++) s[x] = x < rows ? sp[(size_t)(r + 16 * x) * dv] : 0.f;
+  const int chunks = (n + chunk - 1) / chunk;
+  for (int c = 0; c < chunks; c++) {
+    const size_t blk = (size_t)b * max_chunks + c;
+    float* lp = ws_S + (blk * H + h) * dk * dv + cin;
+    const float* pm = ws_P + (blk * H + h) * dk * dk;
+    __syncthreads();                                            // the last chunk's products have read the tiles
+#pragma unroll
+    for (int x = 0; x < DC_ROWS; x++) {
+      if (x < rows) {
+        sh[(r + 16 * x) * 16 + j] = s[x];
+        float* le = lp + (size_t)(r + 16 * x) * dv;
+        acc[x] = *le;                                           // what the chunk makes of a state of zero
+        if (col < dv) *le = s[x];                               // the state in front of this chunk
+      }
+    }
+    for (int e0 = 0; e0 < dk; e0 += ET) {
+      const int ne = min(ET, dk - e0);
+      __syncthreads();                                          // the state's tile is written; the last columns of P are read
+      const int ne4 = (ne + 3) & ~3;
+      for (int idx = threadIdx.x; idx < dk * ne4; idx += 256) {
+        const int i = idx / ne4, ee = idx % ne4;
+        const float x = pm[(size_t)i * dk + min(e0 + ee, dk - 1)];
+        pt[i * ET + ee] = ee < ne ? x : 0.f;
+      }
+      __syncthreads();
+      // four columns of P a turn: the state's four entries serve all rows of the thread, whose sums do not wait for one another
+      const float* sc = sh + e0 * 16 + j;
+      for (int ee = 0; ee < ne4; ee += 4) {
+        const float s0 = sc[ee * 16], s1 = sc[(ee + 1) * 16], s2 = sc[(ee + 2) * 16], s3 = sc[(ee + 3) * 16];
+#pragma unroll
+        for (int x = 0; x < DC_ROWS; x++) {
+          if (x >= rows) break;
+          const float4 p4 = *reinterpret_cast<const float4*>(pt + (r + 16 * x) * ET + ee);
+          acc[x] = fmaf(p4.w, s3, fmaf(p4.z, s2, fmaf(p4.y, s1, fmaf(p4.x, s0, acc[x]))));
+        }
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < DC_ROWS; x++)
+      if (x < rows) s[x] = acc[x];
+  }
+  if (col < dv) {
+#pragma unroll
+    for (int x = 0; x < DC_ROWS; x++)
+      if (x < rows) sp[(size_t)(r + 16 * x) * dv] = s[x];
+  }
 }
 
 #define DELTA_MAX_KEY_DIM 512
@@ -292,41 +396,58 @@ extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, in
   PICO_REQUIRE(chunk >= 0 && (chunk == 0 || (max_chunks > 0 && ws_S && ws_P)), "pico_delta_scan: chunks need their workspace");
   if (num_seqs == 0) return 0;
   // key channels a lane: the fewest of 4, 8, 16, 32 with which at most 4 lanes share a column; beyond 128 channels
-  // more lanes a column
+  // more lanes a column.  Two columns a lane where a head has 32 or more; as many waves (up to four) as the columns ask for.
   int kpl = 4;
   while (kpl < 32 && 4 * kpl < dk) kpl *= 2;
   int KS = 1;
   while (KS * kpl < dk) KS *= 2;
-  const int VC = 64 / KS;
+  const int VC = 64 / KS, DKP = KS * kpl;
+  const int vpl = dv >= 32 ? 2 : 1;
+  const int TB = DKP > 256 ? 8 : 16;
+  const unsigned nblk = (unsigned)(num_seqs * (chunk ? max_chunks : 1));
+  auto waves = [&](int cols) { return min(4, max(1, (cols + VC * vpl - 1) / (VC * vpl))); };
+  auto lds_bytes = [&](int nw) { return (size_t)(3 * TB * DKP + TB * nw * VC * vpl + TB) * sizeof(float); };
+  auto tiles = [&](int cols, int nw) { return (unsigned)((cols + nw * VC * vpl - 1) / (nw * VC * vpl)); };
+  // columns of P in LDS at a time: a multiple of 4, as many as 64 KB hold beside the state's tile
+  const int ET = max(4, min((dk + 3) & ~3, ((16384 - 48) / dk - 16) & ~3));
   const int cols_local = delta ? dv + dk : dv;
-  const dim3 grid_whole(num_seqs, H, (dv + VC - 1) / VC);
-  const dim3 grid_local((unsigned)(num_seqs * (chunk ? max_chunks : 1)), H, (cols_local + VC - 1) / VC);
-  const dim3 grid_from((unsigned)(num_seqs * (chunk ? max_chunks : 1)), H, (dv + VC - 1) / VC);
-  PICO_REQUIRE(grid_local.z <= 65535 && dv <= 65535, "pico_delta_scan: too many value channels");
-#define ARGS(TV) q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens, state_slots, state, out, H, KVH, dk, dv, KS, num_slots, \
+  const int nw_v = waves(dv), nw_l = waves(cols_local);
+  PICO_REQUIRE(tiles(cols_local, nw_l) <= 65535 && (dv + 15) / 16 <= 65535 && ((size_t)dk * dv + 255) / 256 <= 65535,
+               "pico_delta_scan: too many value channels");
+#define ARGS(TV) q, k, (const TV*)v, ldv, g, g_channels, beta, cu_seqlens, state_slots, state, out, H, KVH, dk, dv, KS, TB, num_slots, \
                  chunk, max_chunks, ws_S, ws_P
-#define GO(TV, KPL, D)                                                                            \
-  do {                                                                                            \
-    if (chunk == 0) {                                                                             \
-      delta_scan_kernel<TV, KPL, D, DS_WHOLE><<<grid_whole, 64, 0, stream>>>(ARGS(TV));           \
-    } else {                                                                                      \
-      delta_scan_kernel<TV, KPL, D, DS_LOCAL><<<grid_local, 64, 0, stream>>>(ARGS(TV));           \
-      delta_combine_kernel<D><<<dim3(num_seqs, H, dv), (dk + 63) / 64 * 64, dk * sizeof(float), stream>>>( \
-          cu_seqlens, state_slots, state, ws_S, ws_P, H, dk, dv, num_slots, chunk, max_chunks);   \
-      delta_scan_kernel<TV, KPL, D, DS_FROM><<<grid_from, 64, 0, stream>>>(ARGS(TV));             \
-    }                                                                                             \
+#define GO(TV, KPL, VPL, D)                                                                                                  \
+  do {                                                                                                                       \
+    if (chunk == 0) {                                                                                                        \
+      delta_scan_kernel<TV, KPL, VPL, D, DS_WHOLE><<<dim3(nblk, H, tiles(dv, nw_v)), 64 * nw_v, lds_bytes(nw_v), stream>>>(ARGS(TV)); \
+    } else {                                                                                                                 \
+      delta_scan_kernel<TV, KPL, VPL, D, DS_LOCAL><<<dim3(nblk, H, tiles(cols_local, nw_l)), 64 * nw_l, lds_bytes(nw_l), stream>>>(ARGS(TV)); \
+      if (D)                                                                                                                 \
+        delta_combine_kernel<<<dim3(num_seqs, H, (dv + 15) / 16), 256, ((size_t)dk * (16 + ET) + 48) * sizeof(float), stream>>>( \
+            cu_seqlens, state_slots, state, ws_S, ws_P, H, dk, dv, num_slots, chunk, max_chunks, ET);                        \
+      else                                                                                                                   \
+        decay_combine_kernel<<<dim3(num_seqs, H, (dk * dv + 255) / 256), 256, 0, stream>>>(                                  \
+            cu_seqlens, state_slots, state, ws_S, ws_P, H, dk, dv, num_slots, chunk, max_chunks);                            \
+      delta_scan_kernel<TV, KPL, VPL, D, DS_FROM><<<dim3(nblk, H, tiles(dv, nw_v)), 64 * nw_v, lds_bytes(nw_v), stream>>>(ARGS(TV)); \
+    }                                                                                                                        \
   } while (0)
-#define PICK(TV, D)                    \
-  do {                                 \
-    if (kpl == 4) GO(TV, 4, D);        \
-    else if (kpl == 8) GO(TV, 8, D);   \
-    else if (kpl == 16) GO(TV, 16, D); \
-    else GO(TV, 32, D);                \
+#define PICK2(TV, KPL, D)                  \
+  do {                                     \
+    if (vpl == 2) GO(TV, KPL, 2, D);       \
+    else GO(TV, KPL, 1, D);                \
+  } while (0)
+#define PICK(TV, D)                       \
+  do {                                    \
+    if (kpl == 4) PICK2(TV, 4, D);        \
+    else if (kpl == 8) PICK2(TV, 8, D);   \
+    else if (kpl == 16) PICK2(TV, 16, D); \
+    else PICK2(TV, 32, D);                \
   } while (0)
   if (v_dtype == PICO_DTYPE_F32) { if (delta) PICK(float, true); else PICK(float, false); }
   else if (v_dtype == PICO_DTYPE_BF16) { if (delta) PICK(bf16_t, true); else PICK(bf16_t, false); }
   else PICO_REQUIRE(false, "pico_delta_scan: unknown dtype %d", v_dtype);
 #undef PICK
+#undef PICK2
 #undef GO
 #undef ARGS
   PICO_LAUNCH_CHECK();

@@ -12,10 +12,17 @@
 // float32; a row's sums run in an order that depends on H alone.  One workgroup a row, the row kept in LDS.
 #include "common.h"
 
+#define POSTNORM_MAX_SLABS 8
+
+// The slabs' entries added up in the order of the stack; all loads are issued before the first sum waits for one.
 template <typename T>
 __device__ __forceinline__ float summed(const T* __restrict__ y, int slabs, size_t slab_stride, size_t at) {
-  float v = load_f32(y + at);
-  for (int s = 1; s < slabs; s++) v += load_f32(y + (size_t)s * slab_stride + at);
+  float part[POSTNORM_MAX_SLABS];
+#pragma unroll
+  for (int s = 0; s < POSTNORM_MAX_SLABS; s++) part[s] = load_f32(y + (size_t)min(s, slabs - 1) * slab_stride + at);
+  float v = part[0];
+#pragma unroll
+  for (int s = 1; s < POSTNORM_MAX_SLABS; s++) v += s < slabs ? part[s] : 0.f;
   return v;
 }
 
@@ -99,6 +106,7 @@ extern "C" int pico_norm_add(float* x, const void* a, int a_dtype, int a_slabs, 
                              int T, int H, hipStream_t stream) {
   PICO_REQUIRE(T >= 0 && H > 0 && H * (b ? 2 : 1) <= POSTNORM_MAX_H, "pico_norm_add: a width of 1 to %d (half with two outputs), got %d", POSTNORM_MAX_H, H);
   PICO_REQUIRE(a != nullptr && a_slabs >= 1 && (b == nullptr || (b_slabs >= 1 && wa && wb)), "pico_norm_add: bad operands");
+  PICO_REQUIRE(a_slabs <= POSTNORM_MAX_SLABS && b_slabs <= POSTNORM_MAX_SLABS, "pico_norm_add: at most %d partial sums an output", POSTNORM_MAX_SLABS);
   PICO_REQUIRE((a_slabs == 1 || a_dtype == PICO_DTYPE_F32) && (b == nullptr || b_slabs == 1 || b_dtype == PICO_DTYPE_F32),
                "pico_norm_add: partial sums are float32");
   if (b == nullptr) b_dtype = a_dtype;

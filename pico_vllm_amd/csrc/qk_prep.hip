@@ -18,7 +18,7 @@
 #define QK_NORM_ROW 2
 
 template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_store_kernel(
+__global__ __launch_bounds__(1024) void qk_norm_store_kernel(
     const T* __restrict__ x, int ld, int q_col, int k_col, int v_col, int nq, int nk, int nv, int dk, int dv, int maps,
     int norm_mode, const float* __restrict__ wq, const float* __restrict__ wk, float eps, const float* __restrict__ cos_sin,
     int rot, const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int P,
@@ -95,12 +95,15 @@ extern "C" int pico_qk_norm_store(const void* x, int dtype, int ld, int q_col, i
   PICO_REQUIRE(k_cache == nullptr || (P > 0 && num_pages > 0 && slots), "pico_qk_norm_store: a cache needs pages and slots");
   if (T == 0) return 0;
   if (k_cache == nullptr) { slots = nullptr; v_cache = nullptr; P = 1; num_pages = 0; }
+  // few tokens: a wave a unit, up to sixteen waves, so that a token's units wait for their norms side by side and not one
+  // behind the other; many tokens fill the chip with four waves each
+  const int threads = T >= 64 ? 256 : 64 * min(16, max(4, nq + nk));
   if (dtype == PICO_DTYPE_F32)
-    qk_norm_store_kernel<float><<<T, 256, 0, stream>>>((const float*)x, ld, q_col, k_col, v_col, nq, nk, nv, dk, dv, maps, norm_mode,
+    qk_norm_store_kernel<float><<<T, threads, 0, stream>>>((const float*)x, ld, q_col, k_col, v_col, nq, nk, nv, dk, dv, maps, norm_mode,
                                                        wq, wk, eps, cos_sin, rot, slots, (float*)q_out, (float*)k_cache,
                                                        (float*)v_cache, P, num_pages);
   else if (dtype == PICO_DTYPE_BF16)
-    qk_norm_store_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)x, ld, q_col, k_col, v_col, nq, nk, nv, dk, dv, maps,
+    qk_norm_store_kernel<bf16_t><<<T, threads, 0, stream>>>((const bf16_t*)x, ld, q_col, k_col, v_col, nq, nk, nv, dk, dv, maps,
                                                         norm_mode, wq, wk, eps, cos_sin, rot, slots, (bf16_t*)q_out,
                                                         (bf16_t*)k_cache, (bf16_t*)v_cache, P, num_pages);
   else

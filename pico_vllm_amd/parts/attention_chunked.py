@@ -76,7 +76,8 @@ class ChunkedSinkAttention(Mixer):
         wdt = torch.float32 if any(w.dtype == torch.float32 for w in ws) else ws[0].dtype
         b = None
         if self.proj_bias:
-            b = torch.cat([tensors[n["q_bias"]].float(), tensors[n["k_bias"]].float(), torch.zeros(self.nq)], dim=0).to(device)
+            qb, kb = tensors[n["q_bias"]].float(), tensors[n["k_bias"]].float()
+            b = torch.cat([qb, kb, torch.zeros(self.nq, device=qb.device)], dim=0).to(device)      # the gate has no bias
         self.proj = Linear(torch.cat([t.to(wdt) for t in ws], dim=0).to(device), b)
         self.o = Linear(tensors[n["o"]].to(device))
         self.q_norm = tensors[n["q_norm"]].to(device=device, dtype=torch.float32).contiguous()

@@ -16,11 +16,15 @@ from .spec import CacheSpec, ParamSpec
 # In the bfloat16 engine a step with a prompt portion cuts its sequences into chunks of this many tokens that run side by
 # side (``kernels.delta_scan``); decided from the step's shape alone.  The 32-bit engine walks every sequence whole, so
 # that its sums do not depend on how a prompt was cut.
-CHUNK, CHUNKED_FROM = 64, 128
+# (With the delta rule a chunk's map of the state is a full matrix, and the walk over the chunks, one product a chunk, is
+# a chain of as many steps as a sequence has chunks: longer chunks there.)
+CHUNK, CHUNK_DELTA, CHUNKED_FROM = 64, 128, 128
 
 
-def _chunk(act_dtype: torch.dtype, ctx: StepContext) -> int:
-    return CHUNK if act_dtype == torch.bfloat16 and not ctx.all_decode and ctx.num_tokens >= CHUNKED_FROM else 0
+def _chunk(act_dtype: torch.dtype, ctx: StepContext, delta: bool = False) -> int:
+    if act_dtype != torch.bfloat16 or ctx.all_decode or ctx.num_tokens < CHUNKED_FROM:
+        return 0
+    return CHUNK_DELTA if delta else CHUNK
 
 
 def _conv_state(channels: int, taps: int) -> CacheSpec:
@@ -119,7 +123,7 @@ class GatedDeltaRule(Mixer):
         qn, kn, g, beta = kernels.delta_prep(xc, 0, self.k_col, y, self.b_col, self.a_col, self.a2, self.dt_bias, self.a_log,
                                              self.dk ** -0.5, self.heads, self.qk_heads, self.dk)
         o = kernels.delta_scan(qn, kn, xc[:, self.v_col:], g, beta, ctx.cu_seqlens, ctx.state_slots, state.state, ctx.num_seqs,
-                               self.heads, self.qk_heads, self.dk, self.dv, delta=True, chunk=_chunk(self.act_dtype, ctx))
+                               self.heads, self.qk_heads, self.dk, self.dv, delta=True, chunk=_chunk(self.act_dtype, ctx, delta=True))
         gate = self.g2(y[:, self.g_col:self.g_col + self.gate_rank])
         return kernels.gla_out(o, gate, 0, self.norm_weight, self.norm_eps, self.heads, self.dv, sigmoid_gate=True)
 
