@@ -8,7 +8,7 @@
                                                              continuous batching with prompts cut into portions)
 
   python bench.py --workload designs --layers 4             (Lerazen and Nasedra, each beside the Qwen2.5 shape of equal size,
-                                                             and Dikolix beside Nasedra, at two sizes: decode at batch 1
+                                                             and Dikolix and Vagelix beside Nasedra, at two sizes: decode at batch 1
                                                              and 8, the 2,048-token prefill; --designs nasedra measures
                                                              that design's pairs only)
 
