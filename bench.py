@@ -19,7 +19,7 @@
 
 A step is one decode step of the engine (scheduler, model step from a HIP graph, sampling) at
 batch 8 with every request's context ending at 4096 tokens.  One JSON line goes to stdout:
-decoded tokens a second as ``value`` (K steps between two synchronisations, the contract's clock);
+decoded tokens a second as ``value`` (K steps between two synchronisations: the headline clock);
 ``ms_per_step_median`` from device events around every step; ``prefill`` (one 2,048-token prompt in one
 step, median of device-event times) with its TFLOP/s and its fraction of the bf16 matrix-core peak;
 ``roofline`` (bytes the decode step has to read: every weight once plus the cache of the live requests,
@@ -167,7 +167,7 @@ def decode_point(model_dir, model, dtype, batch, steps, warmup, context=None):
     ctx_start = [r.total_len - 1 for r in eng.requests.values()]
     pool = eng.runner.manager.groups[0].pool
     pages_in_use = pool.num_used
-    # the contract's clock: K steps between two synchronisations; and an event behind every step's launches, whose
+    # the headline clock: K steps between two synchronisations; and an event behind every step's launches, whose
     # distances are the steps' times on the device
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
@@ -460,7 +460,7 @@ def main() -> int:
     ap.add_argument("--no-other", action="store_true", help="skip ``points_other`` (the 7B shape)")
     ap.add_argument("--prefill-only", action="store_true", help="measure only the 2,048-token prefill (for profiling)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
-                    help="with --prefill-only: the prompt's length (2 to 2048; the contract's prefill is of 2,048 tokens)")
+                    help="with --prefill-only: the prompt's length (2 to 2048; the headline prefill is of 2,048 tokens)")
     ap.add_argument("--write-model", metavar="DIR", default=None,
                     help="only write the random-weights model folder to DIR (to reuse with --model) and exit")
     ap.add_argument("--model", default=None, help="measure this model folder (config.json + model.safetensors, any registered "
@@ -470,7 +470,7 @@ def main() -> int:
     ap.add_argument("--designs", default="", help="with --workload designs: only the pairs of these designs (names' beginnings, commas between them)")
     ap.add_argument("--context", type=int, default=4096, help="context length at which the decode steps end")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "sweep", "designs"],
-                    help="decode: the contract's steady decode steps; serve: many requests of mixed lengths at once; "
+                    help="decode: the headline's steady decode steps; serve: many requests of mixed lengths at once; "
                          "long: one prompt of --prompt tokens in portions, then decode at batch 1 and 8 at the context length; "
                          "sweep: decode from context 16 to the context length, the time of a step by context; "
                          "designs: each newer design beside the closest existing model at equal size (--layers of each)")
@@ -660,7 +660,7 @@ def main() -> int:
                 pts[f"decode_b{b}_hbm_frac"] = round(r["gbps"] * 1e9 / HBM_PEAK, 4)
                 log(f"decode batch {b}: {r['tok_s']:.0f} tok/s, {r['ms_per_step']:.3f} ms/step")
             if a.shape == "1.5b" and not a.layers and a.dtype == "bfloat16" and shape_name == SHAPES["1.5b"][0]:
-                # the one figure the reference publishes for this model: 97 tok/s at batch 1 on its authors' card
+                # the one figure the reference publishes for this model: 97 tok/s at batch 1 on its authors' GPU
                 # (README.md:9,43-45 of the reference); other hardware, so a context, not a baseline
                 pts["decode_b1_vs_reference_published"] = round(pts["decode_b1"] / 97.0, 2)
             out["points"] = pts
