@@ -25,7 +25,7 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // grid (T); x: the convolved q | k (columns q_col .., k_col .., KVH heads of dk each); y: the row that holds beta's
 // logits (b_col, H of them) and the low-rank activations (a_col, R of them); a2 [H * dk, R].
 template <typename T>
-__global__ __launch_bounds__(256) void delta_prep_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col,
+__global__ __launch_bounds__(1024) void delta_prep_kernel(const T* __restrict__ x, int ldx, int q_col, int k_col,
                                                          const T* __restrict__ y, int ldy, int b_col, int a_col,
                                                          const T* __restrict__ a2, const float* __restrict__ dt_bias,
                                                          const float* __restrict__ a_log, float qscale, float* __restrict__ qn,
@@ -63,11 +63,12 @@ extern "C" int pico_delta_prep(const void* x, int ldx, int q_col, int k_col, con
                "pico_delta_prep: the rows do not hold what is read");
   if (T == 0) return 0;
   const size_t lds = (size_t)R * sizeof(float);
+  const int threads = T >= 64 ? 256 : 1024;       // few tokens: a thread a decay, so that their sums run side by side
   if (dtype == PICO_DTYPE_F32)
-    delta_prep_kernel<float><<<T, 256, lds, stream>>>((const float*)x, ldx, q_col, k_col, (const float*)y, ldy, b_col, a_col,
+    delta_prep_kernel<float><<<T, threads, lds, stream>>>((const float*)x, ldx, q_col, k_col, (const float*)y, ldy, b_col, a_col,
                                                       (const float*)a2, dt_bias, a_log, qscale, qn, kn, g, beta, H, KVH, dk, R);
   else if (dtype == PICO_DTYPE_BF16)
-    delta_prep_kernel<bf16_t><<<T, 256, lds, stream>>>((const bf16_t*)x, ldx, q_col, k_col, (const bf16_t*)y, ldy, b_col, a_col,
+    delta_prep_kernel<bf16_t><<<T, threads, lds, stream>>>((const bf16_t*)x, ldx, q_col, k_col, (const bf16_t*)y, ldy, b_col, a_col,
                                                        (const bf16_t*)a2, dt_bias, a_log, qscale, qn, kn, g, beta, H, KVH, dk, R);
   else
     PICO_REQUIRE(false, "pico_delta_prep: unknown dtype %d", dtype);
@@ -168,17 +169,24 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict
   const int kvh = h / (H / KVH);
   float* sbase = MODE == DS_WHOLE ? state + (((size_t)slot * H + h) * dk) * dv
                                   : ws_S + (((size_t)blockIdx.x * H + h) * dk) * dv;
+  // The state's loads are unconditional, from addresses clamped into the tensor, and what must not count is cleared in a
+  // loop of its own: a load whose value is selected right behind it is waited for there, and a thread's loads then queue
+  // one behind the other's latency instead of travelling together.
   float S[VPL][KPL];
+  if (MODE != DS_LOCAL) {
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int i = 0; i < KPL; i++)
+        S[j][i] = sbase[(size_t)min(c0 + i, dk - 1) * dv + min(col0 + lcol0 + j * VC, dv - 1)];
+  }
 #pragma unroll
   for (int j = 0; j < VPL; j++) {
     const int col = col0 + lcol0 + j * VC;
 #pragma unroll
     for (int i = 0; i < KPL; i++) {
       if (MODE == DS_LOCAL) S[j][i] = (col >= dv && col < ncols && c0 + i == col - dv) ? 1.f : 0.f;
-      else {
-        const float x = sbase[(size_t)min(c0 + i, dk - 1) * dv + min(col, dv - 1)];
-        S[j][i] = (c0 + i < dk && col < dv) ? x : 0.f;
-      }
+      else S[j][i] = (c0 + i < dk && col < dv) ? S[j][i] : 0.f;
     }
   }
   float gprod[KPL];                                    // DS_LOCAL without the delta rule: the chunk's decays multiplied up
@@ -335,7 +343,8 @@ __global__ __launch_bounds__(256) void delta_combine_kernel(const int* __restric
   float s[DC_ROWS], acc[DC_ROWS];
   float* sp = state + ((size_t)slot * H + h) * dk * dv + cin;
 #pragma unroll
-  for (int x = 0; x < DC_ROWS; x++) s[x] = x < rows ? sp[(size_t)(r + 16 * x) * dv] : 0.f;
+  for (int x = 0; x < DC_ROWS; x++)
+    if (x < rows) s[x] = sp[(size_t)(r + 16 * x) * dv];
   const int chunks = (n + chunk - 1) / chunk;
   for (int c = 0; c < chunks; c++) {
     const size_t blk = (size_t)b * max_chunks + c;
@@ -388,7 +397,7 @@ __global__ __launch_bounds__(256) void delta_combine_kernel(const int* __restric
 
 extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, int ldv, int v_dtype, const float* g,
                                int g_channels, const float* beta, const int* cu_seqlens, const int* state_slots, float* state,
-                               float* out, int num_seqs, int H, int KVH, int dk, int dv, int num_slots, int delta, int chunk,
+                               float* out, int num_seqs, int T, int H, int KVH, int dk, int dv, int num_slots, int delta, int chunk,
                                int max_chunks, float* ws_S, float* ws_P, hipStream_t stream) {
   PICO_REQUIRE(num_seqs >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && dk > 0 && dk <= DELTA_MAX_KEY_DIM && dv > 0 && num_slots > 0,
                "pico_delta_scan: bad sizes (at most %d key channels a head)", DELTA_MAX_KEY_DIM);
@@ -402,10 +411,14 @@ extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, in
   int KS = 1;
   while (KS * kpl < dk) KS *= 2;
   const int VC = 64 / KS, DKP = KS * kpl;
-  const int vpl = dv >= 32 ? 2 : 1;
+  // A step of single tokens is the state read and written once: one column a lane and one wave a workgroup there, four
+  // times the workgroups with a quarter of the loads each in front of the one token's arithmetic.  (A column's sums are
+  // the same whatever the tiling.)
+  const bool few = chunk == 0 && T <= 2 * num_seqs;
+  const int vpl = dv >= 32 && !few ? 2 : 1;
   const int TB = DKP > 256 ? 8 : 16;
   const unsigned nblk = (unsigned)(num_seqs * (chunk ? max_chunks : 1));
-  auto waves = [&](int cols) { return min(4, max(1, (cols + VC * vpl - 1) / (VC * vpl))); };
+  auto waves = [&](int cols) { return few ? 1 : min(4, max(1, (cols + VC * vpl - 1) / (VC * vpl))); };
   auto lds_bytes = [&](int nw) { return (size_t)(3 * TB * DKP + TB * nw * VC * vpl + TB) * sizeof(float); };
   auto tiles = [&](int cols, int nw) { return (unsigned)((cols + nw * VC * vpl - 1) / (nw * VC * vpl)); };
   // columns of P in LDS at a time: a multiple of 4, as many as 64 KB hold beside the state's tile
@@ -457,7 +470,7 @@ extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, in
 // out[t] = norm_groups( (y[t] + D_h x[t]) * silu(z[t]) ) * w: the row of H * dv entries is cut into `groups` equal parts,
 // each over its own root mean square.  grid (T, groups); y float32 [T, H * dv]; x, z columns of wider rows.
 template <typename T>
-__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ x, int ldx,
+__global__ __launch_bounds__(1024) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ x, int ldx,
                                                                const T* __restrict__ z, int ldz, const float* __restrict__ D,
                                                                const float* __restrict__ w, float eps, T* __restrict__ out,
                                                                int H, int dv, int groups) {
@@ -484,10 +497,11 @@ extern "C" int pico_gated_group_norm(const float* y, const void* x, int ldx, con
   if (T == 0) return 0;
   const size_t lds = (size_t)(H * dv / groups) * sizeof(float);
   const dim3 grid(T, groups);
+  const int threads = T >= 64 ? 256 : 1024;       // few tokens: a thread's loads are one turn and travel together
   if (dtype == PICO_DTYPE_F32)
-    gated_group_norm_kernel<float><<<grid, 256, lds, stream>>>(y, (const float*)x, ldx, (const float*)z, ldz, D, w, eps, (float*)out, H, dv, groups);
+    gated_group_norm_kernel<float><<<grid, threads, lds, stream>>>(y, (const float*)x, ldx, (const float*)z, ldz, D, w, eps, (float*)out, H, dv, groups);
   else if (dtype == PICO_DTYPE_BF16)
-    gated_group_norm_kernel<bf16_t><<<grid, 256, lds, stream>>>(y, (const bf16_t*)x, ldx, (const bf16_t*)z, ldz, D, w, eps, (bf16_t*)out, H, dv, groups);
+    gated_group_norm_kernel<bf16_t><<<grid, threads, lds, stream>>>(y, (const bf16_t*)x, ldx, (const bf16_t*)z, ldz, D, w, eps, (bf16_t*)out, H, dv, groups);
   else
     PICO_REQUIRE(false, "pico_gated_group_norm: unknown dtype %d", dtype);
   PICO_LAUNCH_CHECK();

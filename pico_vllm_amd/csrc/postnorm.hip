@@ -28,7 +28,7 @@ __device__ __forceinline__ float summed(const T* __restrict__ y, int slabs, size
 
 // TA, TB: the types of a and b; TO: the type of the copy.
 template <typename TA, typename TB, typename TO>
-__global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, const TA* __restrict__ a, int a_slabs,
+__global__ __launch_bounds__(1024) void norm_add_kernel(float* __restrict__ x, const TA* __restrict__ a, int a_slabs,
                                                        const float* __restrict__ wa, const TB* __restrict__ b, int b_slabs,
                                                        const float* __restrict__ wb, size_t slab_stride,
                                                        const float* __restrict__ w, float eps, TO* __restrict__ copy, int H) {
@@ -113,8 +113,11 @@ extern "C" int pico_norm_add(float* x, const void* a, int a_dtype, int a_slabs, 
   if (copy == nullptr) copy_dtype = PICO_DTYPE_F32;
   if (T == 0) return 0;
   const size_t lds = (size_t)H * sizeof(float) * (b ? 2 : 1);
+  // few rows: as many threads as the row has entries (up to 1,024), so that a thread's loads are one turn and travel
+  // together; many rows fill the chip with four waves each
+  const int threads = T >= 64 ? 256 : min(1024, max(256, (H + 63) / 64 * 64));
 #define LAUNCH(TA, TB, TO)                                                                                                   \
-  norm_add_kernel<TA, TB, TO><<<T, 256, lds, stream>>>(x, (const TA*)a, a_slabs, wa, (const TB*)b, b_slabs, wb,              \
+  norm_add_kernel<TA, TB, TO><<<T, threads, lds, stream>>>(x, (const TA*)a, a_slabs, wa, (const TB*)b, b_slabs, wb,              \
                                                        (size_t)slab_stride, w, eps, (TO*)copy, H)
   const int key = (a_dtype == PICO_DTYPE_BF16 ? 4 : 0) | (b_dtype == PICO_DTYPE_BF16 ? 2 : 0) | (copy_dtype == PICO_DTYPE_BF16 ? 1 : 0);
   PICO_REQUIRE((a_dtype | 1) == 1 && (b_dtype | 1) == 1 && (copy_dtype | 1) == 1, "pico_norm_add: unknown dtype");

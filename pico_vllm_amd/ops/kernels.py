@@ -1428,7 +1428,7 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tenso
     lib = library.core()
     _check(lib, lib.pico_delta_scan(_ptr(q), _ptr(k), _ptr(v), v.stride(0) if T > 1 else v.shape[1], _dt(v), _ptr(g),
                                     1 if g_channels else 0, _ptr(beta), _ptr(cu_seqlens), _ptr(state_slots), _ptr(state), _ptr(out),
-                                    num_seqs, heads, kv_heads, dk, dv, state.shape[0], 1 if delta else 0, chunk, max_chunks, _ptr(ws_s),
+                                    num_seqs, T, heads, kv_heads, dk, dv, state.shape[0], 1 if delta else 0, chunk, max_chunks, _ptr(ws_s),
                                     _ptr(ws_p), _stream()))
     return out
 
