@@ -325,9 +325,11 @@ __global__ __launch_bounds__(256) void decay_combine_kernel(const int* __restric
 
 // The same with the delta rule: S <- P S + L with a full matrix P [dk, dk] a chunk.  grid (sequences, heads,
 // ceil(dv / 16)); a workgroup of 256 threads owns 16 value columns, thread (r, j) the rows r, r + 16, .. of column j.
-// The tile of the state and, ET columns at a time, the chunk's P stand in LDS for the products (P is read from memory
-// once a workgroup, in rows' order).
+// The tile of the state and, ET columns at a time, the chunk's P stand in LDS for the products.  The walk is a chain of
+// as many steps as the sequence has chunks, so a step must not wait for memory: the next tile of P (at most 16 floats a
+// thread) and the next chunk's L travel in registers while this tile's products run.
 #define DC_ROWS 32          // rows a thread: 512 key channels at most
+#define DC_TILE 16          // floats of a tile of P a thread holds on their way to LDS
 __global__ __launch_bounds__(256) void delta_combine_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
                                                             float* __restrict__ state, float* __restrict__ ws_S,
                                                             const float* __restrict__ ws_P, int H, int dk, int dv, int num_slots,
@@ -340,38 +342,71 @@ __global__ __launch_bounds__(256) void delta_combine_kernel(const int* __restric
   const int slot = state_slots[b], n = cu_seqlens[b + 1] - cu_seqlens[b];
   if (slot < 0 || slot >= num_slots || n <= 0) return;          // the whole workgroup
   const int rows = (dk - r + 15) / 16;                          // rows r, r + 16, .. below dk
-  float s[DC_ROWS], acc[DC_ROWS];
+  const int ntile = (dk + ET - 1) / ET;
+  const int chunks = (n + chunk - 1) / chunk;
+  float s[DC_ROWS], acc[DC_ROWS], lnext[DC_ROWS], pre[DC_TILE];
   float* sp = state + ((size_t)slot * H + h) * dk * dv + cin;
+  // every load is unconditional, from a clamped address; what must not count is never used
+  auto load_local = [&](int c) {
+    const float* lp = ws_S + ((((size_t)b * max_chunks + c) * H + h) * dk) * dv + cin;
+#pragma unroll
+    for (int x = 0; x < DC_ROWS; x++)
+      if (x < rows) lnext[x] = lp[(size_t)min(r + 16 * x, dk - 1) * dv];
+  };
+  // ET is a power of two: a thread's place in a tile is a shift and a mask away
+  const int eshift = 31 - __clz(ET);
+  auto fetch_tile = [&](int c, int tile) {
+    const float* pm = ws_P + ((((size_t)b * max_chunks + c) * H + h) * dk) * dk;
+    const int e0 = tile * ET;
+#pragma unroll
+    for (int m = 0; m < DC_TILE; m++) {
+      const int idx = (int)threadIdx.x + 256 * m, i = idx >> eshift, ee = idx & (ET - 1);
+      pre[m] = pm[(size_t)min(i, dk - 1) * dk + min(e0 + ee, dk - 1)];
+    }
+  };
+  auto store_tile = [&](int tile) {
+    const int e0 = tile * ET, ne = min(ET, dk - e0);
+#pragma unroll
+    for (int m = 0; m < DC_TILE; m++) {
+      const int idx = (int)threadIdx.x + 256 * m, i = idx >> eshift, ee = idx & (ET - 1);
+      if (i < dk) pt[idx] = ee < ne ? pre[m] : 0.f;
+    }
+  };
 #pragma unroll
   for (int x = 0; x < DC_ROWS; x++)
     if (x < rows) s[x] = sp[(size_t)(r + 16 * x) * dv];
-  const int chunks = (n + chunk - 1) / chunk;
+  load_local(0);
+  fetch_tile(0, 0);
   for (int c = 0; c < chunks; c++) {
-    const size_t blk = (size_t)b * max_chunks + c;
-    float* lp = ws_S + (blk * H + h) * dk * dv + cin;
-    const float* pm = ws_P + (blk * H + h) * dk * dk;
+    float* lp = ws_S + ((((size_t)b * max_chunks + c) * H + h) * dk) * dv + cin;
     __syncthreads();                                            // the last chunk's products have read the tiles
 #pragma unroll
     for (int x = 0; x < DC_ROWS; x++) {
       if (x < rows) {
         sh[(r + 16 * x) * 16 + j] = s[x];
-        float* le = lp + (size_t)(r + 16 * x) * dv;
-        acc[x] = *le;                                           // what the chunk makes of a state of zero
-        if (col < dv) *le = s[x];                               // the state in front of this chunk
+        acc[x] = lnext[x];                                      // what the chunk makes of a state of zero
       }
     }
-    for (int e0 = 0; e0 < dk; e0 += ET) {
-      const int ne = min(ET, dk - e0);
-      __syncthreads();                                          // the state's tile is written; the last columns of P are read
-      const int ne4 = (ne + 3) & ~3;
-      for (int idx = threadIdx.x; idx < dk * ne4; idx += 256) {
-        const int i = idx / ne4, ee = idx % ne4;
-        const float x = pm[(size_t)i * dk + min(e0 + ee, dk - 1)];
-        pt[i * ET + ee] = ee < ne ? x : 0.f;
+    for (int tile = 0; tile < ntile; tile++) {
+      const int e0 = tile * ET, ne4 = (min(ET, dk - e0) + 3) & ~3;
+      if (tile > 0) __syncthreads();                            // the last tile's products have read it
+      store_tile(tile);
+      __syncthreads();                                          // the state's tile and this tile of P are written
+      // everything that goes to or comes from memory is issued here, behind the barrier (which waits for what is under
+      // way) and in front of the products, under which it travels
+      if (tile + 1 < ntile) fetch_tile(c, tile + 1);
+      else if (c + 1 < chunks) fetch_tile(c + 1, 0);
+      if (tile == 0) {
+        if (col < dv) {
+#pragma unroll
+          for (int x = 0; x < DC_ROWS; x++)
+            if (x < rows) lp[(size_t)(r + 16 * x) * dv] = s[x];  // the state in front of this chunk
+        }
+        if (c + 1 < chunks) load_local(c + 1);
       }
-      __syncthreads();
       // four columns of P a turn: the state's four entries serve all rows of the thread, whose sums do not wait for one another
       const float* sc = sh + e0 * 16 + j;
+#pragma unroll 2
       for (int ee = 0; ee < ne4; ee += 4) {
         const float s0 = sc[ee * 16], s1 = sc[(ee + 1) * 16], s2 = sc[(ee + 2) * 16], s3 = sc[(ee + 3) * 16];
 #pragma unroll
@@ -421,8 +456,9 @@ extern "C" int pico_delta_scan(const float* q, const float* k, const void* v, in
   auto waves = [&](int cols) { return few ? 1 : min(4, max(1, (cols + VC * vpl - 1) / (VC * vpl))); };
   auto lds_bytes = [&](int nw) { return (size_t)(3 * TB * DKP + TB * nw * VC * vpl + TB) * sizeof(float); };
   auto tiles = [&](int cols, int nw) { return (unsigned)((cols + nw * VC * vpl - 1) / (nw * VC * vpl)); };
-  // columns of P in LDS at a time: a multiple of 4, as many as 64 KB hold beside the state's tile
-  const int ET = max(4, min((dk + 3) & ~3, ((16384 - 48) / dk - 16) & ~3));
+  // columns of P in LDS at a time: a power of two from 4, as many as a workgroup's threads carry 16 floats each of
+  int ET = 4;
+  while (2 * ET * dk <= 256 * DC_TILE && ET < dk) ET *= 2;
   const int cols_local = delta ? dv + dk : dv;
   const int nw_v = waves(dv), nw_l = waves(cols_local);
   PICO_REQUIRE(tiles(cols_local, nw_l) <= 65535 && (dv + 15) / 16 <= 65535 && ((size_t)dk * dv + 255) / 256 <= 65535,

@@ -17,8 +17,8 @@ from .spec import CacheSpec, ParamSpec
 # side (``kernels.delta_scan``); decided from the step's shape alone.  The 32-bit engine walks every sequence whole, so
 # that its sums do not depend on how a prompt was cut.
 # (With the delta rule a chunk's map of the state is a full matrix, and the walk over the chunks, one product a chunk, is
-# a chain of as many steps as a sequence has chunks: longer chunks there.)
-CHUNK, CHUNK_DELTA, CHUNKED_FROM = 64, 128, 128
+# a chain of as many steps as a sequence has chunks; longer chunks shorten it and take as much from the two passes.)
+CHUNK, CHUNK_DELTA, CHUNKED_FROM = 64, 64, 128
 
 
 def _chunk(act_dtype: torch.dtype, ctx: StepContext, delta: bool = False) -> int:
