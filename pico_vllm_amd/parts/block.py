@@ -204,7 +204,8 @@ class PostNormBlock(Block):
         if pending is not None:                                   # a block in front that hands a delta on
             for d in (pending if pending.dim() == 3 else (pending,)):
                 kernels.residual_add(resid, d)
-            ctx.shared.pop("stream_copy", None)
+            from .norm import STREAM_COPY
+            ctx.shared.pop(STREAM_COPY, None)                     # the stream's copy in the activations' type is stale now
         h = self._rows(resid, ctx)
         pair = getattr(p["mixer"], "forward_pair", None)
         if pair is not None:

@@ -192,7 +192,7 @@ class DecoderModel:
         for i, e in enumerate(self.spec.run_order):
             if e.add_input:
                 kernels.residual_add(resid, entered)       # what is pending joins later; the sums are float32
-                ctx.shared.pop("stream_copy", None)            # a copy of the stream in the activations' dtype is stale now
+                ctx.shared.pop(norm.STREAM_COPY, None)         # a copy of the stream in the activations' dtype is stale now
             # a run that names another run's cache reads it and stores nothing of its own
             resid, pending = self.layers[e.layer].forward(resid, pending, ctx,
                                                           storage.layer(self.spec.cache_id(i), read_only=e.cache_of is not None))

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import plain_vagelix as P
-from vagelix_configs import CONFIGS, attention, config, mamba2, model_dir, parallel, tensors_of
+from vagelix_configs import CONFIGS, model_dir, tensors_of
 
 F = torch.float64
 
